@@ -1,0 +1,95 @@
+// Shared device helpers for the gfx950 kernels: wave64 reductions, bf16 <-> f32
+// conversion (round to nearest even), typed loads/stores, launch checking.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_bf16.h>
+#include <stdint.h>
+
+#define EI_WAVE 64
+#define EI_PAGE 64  // tokens of one sequence that a cache page holds
+
+// dtype codes of the C interface
+#define EI_F32 0
+#define EI_BF16 1
+
+typedef uint16_t bf16_t;  // raw bfloat16 bits
+
+namespace ei {
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(static_cast<uint32_t>(v) << 16);
+}
+
+// round to nearest even; NaN stays NaN
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return static_cast<bf16_t>((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return static_cast<bf16_t>(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ float to_f32(T v);
+template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return bf16_to_f32(v); }
+
+template <typename T> __device__ __forceinline__ T from_f32(float v);
+template <> __device__ __forceinline__ float from_f32<float>(float v) { return v; }
+template <> __device__ __forceinline__ bf16_t from_f32<bf16_t>(float v) { return f32_to_bf16(v); }
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, EI_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1)
+    v = fmaxf(v, __shfl_xor(v, offset, EI_WAVE));
+  return v;
+}
+
+// Sum over a block of `blockDim.x` threads (a multiple of 64, at most 1024).
+// `scratch` holds at least 16 floats.  Every thread gets the total.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
+  const int waves = blockDim.x / EI_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int i = 0; i < waves; ++i) total += scratch[i];
+  return total;
+}
+
+}  // namespace ei
+
+// Host side ---------------------------------------------------------------
+// Each kernel library is one translation unit and carries its own message buffer.
+#include <string.h>
+static thread_local char ei_error_text[512];
+static inline void ei_set_error(const char* message) {
+  strncpy(ei_error_text, message, sizeof(ei_error_text) - 1);
+  ei_error_text[sizeof(ei_error_text) - 1] = 0;
+}
+extern "C" const char* ei_last_error() { return ei_error_text; }
+
+#define EI_REQUIRE(cond, msg)       \
+  do {                              \
+    if (!(cond)) {                  \
+      ei_set_error(msg);            \
+      return -1;                    \
+    }                               \
+  } while (0)
+
+#define EI_LAUNCH_CHECK()                         \
+  do {                                            \
+    hipError_t e_ = hipGetLastError();            \
+    if (e_ != hipSuccess) {                       \
+      ei_set_error(hipGetErrorString(e_));        \
+      return static_cast<int>(e_);                \
+    }                                             \
+    return 0;                                     \
+  } while (0)

@@ -1,0 +1,291 @@
+"""ctypes bindings of the HIP kernel libraries.
+
+Each function takes torch tensors that live on the GPU, checks what the kernel
+assumes about them (device, dtype, contiguity, sizes) and launches on torch's
+current stream.  A library is loaded (and compiled, when it is not yet) the first
+time one of its functions is called.  There is no other implementation behind
+these functions: if a library cannot be built or loaded the call raises.
+"""
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_float, c_int, c_longlong, c_ulonglong, c_void_p
+from typing import Dict, Optional
+
+import torch
+
+from . import build
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+PAGE_TOKENS = 64
+
+_SIGNATURES = {
+    "rowwise": {
+        "ei_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
+        "ei_add_rmsnorm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
+                           c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
+        "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int,
+                      c_void_p],
+    },
+    "rope_store": {
+        "ei_qk_norm_rope_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_float,
+                                  c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int, c_void_p,
+                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                  c_void_p],
+    },
+    "attention_generic": {
+        "ei_attn_heads_per_block": [c_int],
+        "ei_attn_positions_per_item": [c_int],
+        "ei_attention": [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                         c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                         c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
+    },
+    "gemm_f32": {
+        "ei_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_longlong, c_longlong,
+                        c_longlong, c_void_p],
+    },
+    "sampling": {
+        "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
+        "ei_sample": [c_void_p, c_int, c_int, c_float, c_float, c_int, c_ulonglong, c_void_p,
+                      c_void_p, c_void_p, c_void_p, c_void_p],
+    },
+}
+
+_loaded: Dict[str, ctypes.CDLL] = {}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def library(name: str) -> ctypes.CDLL:
+    lib = _loaded.get(name)
+    if lib is not None:
+        return lib
+    path = build.build_library(name)
+    try:
+        lib = ctypes.CDLL(str(path))
+    except OSError as error:
+        raise KernelError(f"cannot load kernel library {path}: {error}") from error
+    for symbol, argtypes in _SIGNATURES.get(name, {}).items():
+        function = getattr(lib, symbol)
+        function.argtypes = argtypes
+        function.restype = c_int
+    lib.ei_last_error.restype = ctypes.c_char_p
+    _loaded[name] = lib
+    return lib
+
+
+def loaded_libraries():
+    return sorted(_loaded)
+
+
+def _check(lib, status: int, what: str) -> None:
+    if status != 0:
+        message = lib.ei_last_error().decode(errors="replace")
+        raise KernelError(f"{what}: {message} (status {status})")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _gpu(tensor: torch.Tensor, name: str, dtype=None) -> int:
+    if not tensor.is_cuda:
+        raise KernelError(f"{name} must live on the GPU")
+    if not tensor.is_contiguous():
+        raise KernelError(f"{name} must be contiguous")
+    if dtype is not None and tensor.dtype != dtype:
+        raise KernelError(f"{name} must be {dtype}, got {tensor.dtype}")
+    return tensor.data_ptr()
+
+
+def _code(tensor: torch.Tensor, name: str) -> int:
+    try:
+        return _DTYPE_CODE[tensor.dtype]
+    except KeyError:
+        raise KernelError(f"{name} has unsupported dtype {tensor.dtype}") from None
+
+
+def _splits(tensor: torch.Tensor, rows: int, width: int, name: str):
+    """(nsplit, stride) of a [rows, width] or [nsplit, rows, width] tensor."""
+    if tensor.dim() == 2 and tuple(tensor.shape) == (rows, width):
+        return 1, 0
+    if tensor.dim() == 3 and tuple(tensor.shape[1:]) == (rows, width):
+        return tensor.shape[0], rows * width
+    raise KernelError(f"{name} must be [{rows}, {width}] or [splits, {rows}, {width}], "
+                      f"got {list(tensor.shape)}")
+
+
+# ---------------------------------------------------------------------------
+def embed_gather(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor) -> None:
+    lib = library("rowwise")
+    n = ids.numel()
+    vocab, hidden = table.shape
+    if tuple(out.shape) != (n, hidden):
+        raise KernelError(f"embed_gather: out must be [{n}, {hidden}], got {list(out.shape)}")
+    status = lib.ei_embed_gather(_gpu(ids, "ids", torch.int32), _gpu(table, "table"),
+                                 _code(table, "table"), _gpu(out, "out", torch.float32), n,
+                                 hidden, vocab, _stream())
+    _check(lib, status, "embed_gather")
+
+
+def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                eps: float, out: torch.Tensor, rows: Optional[torch.Tensor] = None,
+                write_residual: bool = True) -> None:
+    """residual [R, H] float32 (+= sum of delta splits, stored back unless told not
+    to); out[i] = rmsnorm(residual[rows[i] if rows else i]) * weight."""
+    lib = library("rowwise")
+    total_rows, hidden = residual.shape
+    n = out.shape[0]
+    if out.dim() != 2 or out.shape[1] != hidden:
+        raise KernelError(f"add_rmsnorm: out must be [*, {hidden}], got {list(out.shape)}")
+    if weight.numel() != hidden:
+        raise KernelError(f"add_rmsnorm: weight must have {hidden} elements")
+    if rows is None and n != total_rows:
+        raise KernelError("add_rmsnorm: out and residual row counts differ")
+    if rows is not None and rows.numel() != n:
+        raise KernelError("add_rmsnorm: rows and out row counts differ")
+    nsplit, stride, delta_ptr, delta_code = 0, 0, None, F32
+    if delta is not None:
+        nsplit, stride = _splits(delta, total_rows, hidden, "delta")
+        delta_ptr, delta_code = _gpu(delta, "delta"), _code(delta, "delta")
+    status = lib.ei_add_rmsnorm(
+        _gpu(residual, "residual", torch.float32), delta_ptr, delta_code, nsplit, stride,
+        None if rows is None else _gpu(rows, "rows", torch.int32),
+        _gpu(weight, "weight", torch.float32), float(eps), _gpu(out, "out"), _code(out, "out"), n,
+        hidden, int(write_residual), _stream())
+    _check(lib, status, "add_rmsnorm")
+
+
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    lib = library("rowwise")
+    n, inter = out.shape
+    nsplit, stride = _splits(gate_up, n, 2 * inter, "gate_up")
+    status = lib.ei_swiglu(_gpu(gate_up, "gate_up"), _code(gate_up, "gate_up"), nsplit, stride,
+                           _gpu(out, "out"), _code(out, "out"), n, inter, _stream())
+    _check(lib, status, "swiglu")
+
+
+def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, eps, rope_table, row_pos, row_seq, page_table,
+                       q_out, k_pages, v_pages, n_heads, n_kv_heads, head_dim,
+                       write_cache=True) -> None:
+    lib = library("rope_store")
+    n = q_out.shape[0]
+    width = (n_heads + 2 * n_kv_heads) * head_dim
+    nsplit, stride = _splits(qkv, n, width, "qkv")
+    if tuple(q_out.shape) != (n, n_heads * head_dim):
+        raise KernelError("qk_norm_rope_store: q_out has the wrong shape")
+    if row_pos.numel() < n or row_seq.numel() < n:
+        raise KernelError("qk_norm_rope_store: row metadata shorter than the rows")
+    max_pos = 0
+    if rope_table is not None:
+        if rope_table.dim() != 2 or rope_table.shape[1] != head_dim:
+            raise KernelError("qk_norm_rope_store: rope table must be [positions, head_dim]")
+        max_pos = rope_table.shape[0]
+    if write_cache:
+        expect = (n_kv_heads, PAGE_TOKENS, head_dim)
+        if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
+            raise KernelError(f"qk_norm_rope_store: pages must be [*, {expect}]")
+        if k_pages.dtype != q_out.dtype or v_pages.dtype != q_out.dtype:
+            raise KernelError("qk_norm_rope_store: cache and q_out dtypes differ")
+    status = lib.ei_qk_norm_rope_store(
+        _gpu(qkv, "qkv"), _code(qkv, "qkv"), nsplit, stride,
+        None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
+        None if k_norm_w is None else _gpu(k_norm_w, "k_norm", torch.float32), float(eps),
+        None if rope_table is None else _gpu(rope_table, "rope_table", torch.float32), max_pos,
+        _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+        _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
+        _gpu(q_out, "q_out"), _gpu(k_pages, "k_pages") if write_cache else None,
+        _gpu(v_pages, "v_pages") if write_cache else None, _code(q_out, "q_out"), n, n_heads,
+        n_kv_heads, head_dim, int(write_cache), _stream())
+    _check(lib, status, "qk_norm_rope_store")
+
+
+def attention_heads_per_block(group: int) -> int:
+    return library("attention_generic").ei_attn_heads_per_block(group)
+
+
+def attention_positions_per_item(group: int) -> int:
+    return library("attention_generic").ei_attn_positions_per_item(group)
+
+
+def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos, row_seq,
+              page_table, out, n_heads, n_kv_heads, head_dim, window=None, scale=None,
+              n_splits=1, part_o=None, part_ml=None) -> None:
+    """Generic causal attention over the paged cache (see attention_generic.hip)."""
+    lib = library("attention_generic")
+    n = q.shape[0]
+    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
+        raise KernelError("attention: q and out must be [rows, heads * head_dim]")
+    expect = (n_kv_heads, PAGE_TOKENS, head_dim)
+    if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
+        raise KernelError(f"attention: pages must be [*, {expect}]")
+    if not (q.dtype == k_pages.dtype == v_pages.dtype == out.dtype):
+        raise KernelError("attention: q, cache and out dtypes differ")
+    if item_seq.numel() < n_items or item_row0.numel() < n_items or item_npos.numel() < n_items:
+        raise KernelError("attention: work item arrays shorter than n_items")
+    if n_splits > 1:
+        need_o = n * n_heads * n_splits * head_dim
+        if part_o is None or part_ml is None or part_o.numel() < need_o \
+                or part_ml.numel() < n * n_heads * n_splits * 2:
+            raise KernelError("attention: split scratch missing or too small")
+    if scale is None:
+        scale = head_dim ** -0.5
+    status = lib.ei_attention(
+        _gpu(q, "q"), _gpu(k_pages, "k_pages"), _gpu(v_pages, "v_pages"), _code(q, "q"),
+        _gpu(item_seq, "item_seq", torch.int32), _gpu(item_row0, "item_row0", torch.int32),
+        _gpu(item_npos, "item_npos", torch.int32), n_items, _gpu(row_pos, "row_pos", torch.int32),
+        _gpu(row_seq, "row_seq", torch.int32), _gpu(page_table, "page_table", torch.int32),
+        page_table.shape[-1], _gpu(out, "out"),
+        None if part_o is None else _gpu(part_o, "part_o", torch.float32),
+        None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
+        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, _stream())
+    _check(lib, status, "attention")
+
+
+def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[M, N] = a[M, K] . w[N, K]^T in float32."""
+    lib = library("gemm_f32")
+    m, k = a.shape
+    n = w.shape[0]
+    if w.shape[1] != k or tuple(out.shape) != (m, n):
+        raise KernelError(f"gemm_f32: shapes {list(a.shape)} x {list(w.shape)}^T -> "
+                          f"{list(out.shape)} do not agree")
+    status = lib.ei_gemm_f32(_gpu(a, "a", torch.float32), _gpu(w, "w", torch.float32),
+                             _gpu(out, "out", torch.float32), m, n, k, k, k, n, _stream())
+    _check(lib, status, "gemm_f32")
+
+
+def argmax(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None) -> None:
+    lib = library("sampling")
+    rows, vocab = logits.shape
+    if tokens.numel() < rows:
+        raise KernelError("argmax: tokens shorter than the rows")
+    status = lib.ei_argmax(_gpu(logits, "logits", torch.float32), rows, vocab,
+                           _gpu(tokens, "tokens", torch.int32),
+                           None if probabilities is None
+                           else _gpu(probabilities, "probabilities", torch.float32), _stream())
+    _check(lib, status, "argmax")
+
+
+def sample(logits, temperature, top_p, top_k, seed, streams, counters, tokens,
+           probabilities=None) -> None:
+    lib = library("sampling")
+    rows, vocab = logits.shape
+    if tokens.numel() < rows or streams.numel() < rows or counters.numel() < rows:
+        raise KernelError("sample: per-row arrays shorter than the rows")
+    status = lib.ei_sample(_gpu(logits, "logits", torch.float32), rows, vocab, float(temperature),
+                           float(top_p), int(top_k), int(seed) & (2**64 - 1),
+                           _gpu(streams, "streams", torch.int32),
+                           _gpu(counters, "counters", torch.int32),
+                           _gpu(tokens, "tokens", torch.int32),
+                           None if probabilities is None
+                           else _gpu(probabilities, "probabilities", torch.float32), _stream())
+    _check(lib, status, "sample")
+
+
+# ---------------------------------------------------------------------------
+def has_skinny_gemm() -> bool:
+    return "gemm_bf16" in build.available_libraries()

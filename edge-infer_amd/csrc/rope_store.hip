@@ -1,0 +1,139 @@
+// Fused per-head q/k RMSNorm -> rotary encoding -> cache store.
+//
+// One wave per (row, head) over the packed projection [N, Q + 2*KV]: query heads
+// are normed, rotated and written to q_out; key heads are normed, rotated and
+// written to the cache page of (sequence, position); value heads are copied to
+// the cache.  Sum of squares, inverse RMS, angles' sine/cosine (a float32 table)
+// and the rotation are float32; one rounding to the storage type.
+//
+// Formulas of the reference: norm before rotation,
+// runtime/include/execution/decoder.hpp:125-140; rotate-half pairs (i, i + d/2),
+// x' = x cos - y sin, y' = x sin + y cos, operators/src/cuda/execution.cu:79-122;
+// keys stored after norm and rotation, values raw, decoder.hpp:137-140.
+#include "common.cuh"
+
+namespace {
+
+constexpr int kMaxPairsPerLane = 4;  // head_dim up to 512
+
+template <typename TI, typename TO>
+__global__ void qk_norm_rope_store_kernel(
+    const TI* __restrict__ qkv, int nsplit, size_t split_stride,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ rope_table,  // [max_pos, D]: cos[D/2] then sin[D/2]; null: none
+    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_seq,
+    const int32_t* __restrict__ page_table, int table_width,
+    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
+    int N, int nq, int nkv, int D, int write_cache) {
+  const int heads = nq + 2 * nkv;
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
+  const int lane = threadIdx.x % EI_WAVE;
+  if (wave >= N * heads) return;
+  const int row = wave / heads, head = wave % heads;
+  const int seq = row_seq[row];
+  if (seq < 0) return;  // padding row
+  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  if (!is_q && !write_cache) return;
+  const int pos = row_pos[row];
+  const int half = D / 2;
+  const size_t width = static_cast<size_t>(nq + 2 * nkv) * D;
+  const TI* src = qkv + static_cast<size_t>(row) * width + static_cast<size_t>(head) * D;
+
+  float x[kMaxPairsPerLane], y[kMaxPairsPerLane];
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < kMaxPairsPerLane; ++j) {
+    const int i = lane + j * EI_WAVE;
+    x[j] = 0.f;
+    y[j] = 0.f;
+    if (i < half) {
+      for (int s = 0; s < nsplit; ++s) {
+        x[j] += ei::to_f32<TI>(src[s * split_stride + i]);
+        y[j] += ei::to_f32<TI>(src[s * split_stride + i + half]);
+      }
+      sum += x[j] * x[j] + y[j] * y[j];
+    }
+  }
+
+  TO* dst;
+  if (is_q) {
+    dst = q_out + static_cast<size_t>(row) * nq * D + static_cast<size_t>(head) * D;
+  } else {
+    const int page = page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE];
+    if (page < 0) return;
+    const int g = is_k ? head - nq : head - nq - nkv;
+    TO* base = is_k ? k_pages : v_pages;
+    dst = base + ((static_cast<size_t>(page) * nkv + g) * EI_PAGE + pos % EI_PAGE) * D;
+  }
+
+  const float* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+  float inv = 1.f;
+  if (norm_w) {
+    sum = ei::wave_sum(sum);
+    inv = rsqrtf(sum / static_cast<float>(D) + eps);
+  }
+  const bool rotate = rope_table != nullptr && (is_q || is_k);
+  const float* trig = rotate ? rope_table + static_cast<size_t>(pos) * D : nullptr;
+#pragma unroll
+  for (int j = 0; j < kMaxPairsPerLane; ++j) {
+    const int i = lane + j * EI_WAVE;
+    if (i < half) {
+      float a = x[j], b = y[j];
+      if (norm_w) {
+        a = (a * inv) * norm_w[i];
+        b = (b * inv) * norm_w[i + half];
+      }
+      if (rotate) {
+        const float c = trig[i], s = trig[i + half];
+        const float ra = a * c - b * s;
+        const float rb = a * s + b * c;
+        a = ra;
+        b = rb;
+      }
+      dst[i] = ei::from_f32<TO>(a);
+      dst[i + half] = ei::from_f32<TO>(b);
+    }
+  }
+}
+
+}  // namespace
+
+// qkv: [nsplit][N, (nq + 2 nkv) * D] of in_dtype.  q_out: [N, nq * D] of out_dtype.
+// k_pages / v_pages: [n_pages, nkv, 64, D] of out_dtype for this cache entry.
+// page_table: int32 [n_seqs, table_width], logical page -> physical page.
+extern "C" int ei_qk_norm_rope_store(
+    const void* qkv, int in_dtype, int nsplit, long long split_stride, const float* q_norm_w,
+    const float* k_norm_w, float eps, const float* rope_table, int max_pos,
+    const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table, int table_width,
+    void* q_out, void* k_pages, void* v_pages, int out_dtype, int N, int nq, int nkv, int D,
+    int write_cache, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && nq > 0 && nkv > 0 && D > 0, "qk_norm_rope_store: sizes must be positive");
+  EI_REQUIRE(D % 2 == 0, "qk_norm_rope_store: head_dim must be even");
+  EI_REQUIRE(D / 2 <= kMaxPairsPerLane * EI_WAVE, "qk_norm_rope_store: head_dim above 512");
+  EI_REQUIRE(qkv && row_pos && row_seq && q_out, "qk_norm_rope_store: null pointer");
+  EI_REQUIRE(!write_cache || (k_pages && v_pages && page_table && table_width > 0),
+             "qk_norm_rope_store: cache pointers missing");
+  EI_REQUIRE(nsplit >= 1, "qk_norm_rope_store: nsplit must be at least 1");
+  (void)max_pos;
+  const int heads = nq + 2 * nkv;
+  const long long waves = static_cast<long long>(N) * heads;
+  const int threads = 256;
+  const long long blocks = (waves * EI_WAVE + threads - 1) / threads;
+  EI_REQUIRE(blocks < (1ll << 31), "qk_norm_rope_store: too many rows");
+  const size_t ss = static_cast<size_t>(split_stride);
+#define EI_ROPE_LAUNCH(TI, TO)                                                                   \
+  qk_norm_rope_store_kernel<TI, TO><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(      \
+      static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, rope_table, row_pos,     \
+      row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),      \
+      static_cast<TO*>(v_pages), N, nq, nkv, D, write_cache)
+  if (in_dtype == EI_F32 && out_dtype == EI_F32)
+    EI_ROPE_LAUNCH(float, float);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
+    EI_ROPE_LAUNCH(float, bf16_t);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
+    EI_ROPE_LAUNCH(bf16_t, bf16_t);
+  else
+    EI_REQUIRE(false, "qk_norm_rope_store: unsupported dtype combination");
+#undef EI_ROPE_LAUNCH
+  EI_LAUNCH_CHECK();
+}

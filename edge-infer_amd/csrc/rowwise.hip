@@ -1,0 +1,165 @@
+// Row-wise kernels of the decoder step: embedding gather, fused residual-add +
+// RMSNorm (optionally on gathered rows), SiLU-gate product.  The residual stream is
+// float32 in both precisions; sums of squares, the inverse RMS and the products
+// are float32 and the result is rounded once to the output type.
+//
+// Formulas: operators/src/cuda/execution.cu:67-78 (gather),
+// operators/src/cuda/rms_norm_cuda.cu:19-101 (x * rsqrt(mean(x^2) + eps) * w),
+// operators/src/cuda/silu_cuda.cu:44-56 (silu(gate) * up) of the reference.
+#include "common.cuh"
+
+namespace {
+
+template <typename T>
+__global__ void embed_gather_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
+                                    float* __restrict__ out, int H, int V) {
+  const int row = blockIdx.x;
+  const int id = ids[row];
+  float* dst = out + static_cast<size_t>(row) * H;
+  if (id < 0 || id >= V) {
+    for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = 0.f;
+    return;
+  }
+  const T* src = table + static_cast<size_t>(id) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = ei::to_f32<T>(src[i]);
+}
+
+// One block per output row.  x = residual[src] (+ sum over splits of delta[s][src]);
+// optionally stored back; out[row] = x * rsqrt(mean(x^2) + eps) * weight.
+template <typename TD, typename TO, bool HAS_DELTA>
+__global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                   int nsplit, size_t split_stride,
+                                   const int32_t* __restrict__ rows,
+                                   const float* __restrict__ weight, float eps,
+                                   TO* __restrict__ out, int H, int write_residual) {
+  extern __shared__ float row_values[];
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const int src = rows ? rows[row] : row;
+  if (src < 0) {  // padding row of a fixed-size batch: defined output, nothing else touched
+    for (int i = threadIdx.x; i < H; i += blockDim.x)
+      out[static_cast<size_t>(row) * H + i] = ei::from_f32<TO>(0.f);
+    return;
+  }
+  float* res = residual + static_cast<size_t>(src) * H;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x = res[i];
+    if (HAS_DELTA) {
+      const TD* d = delta + static_cast<size_t>(src) * H + i;
+      for (int s = 0; s < nsplit; ++s) x += ei::to_f32<TD>(d[s * split_stride]);
+      if (write_residual) res[i] = x;
+    }
+    row_values[i] = x;
+    sum += x * x;
+  }
+  const float total = ei::block_sum(sum, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(H) + eps);
+  TO* dst = out + static_cast<size_t>(row) * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    dst[i] = ei::from_f32<TO>((row_values[i] * inv) * weight[i]);
+}
+
+template <typename TI, typename TO>
+__global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
+                              TO* __restrict__ out, int I, size_t total) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t idx = start; idx < total; idx += step) {
+    const size_t row = idx / I, col = idx % I;
+    const TI* g = gate_up + row * 2 * I + col;
+    float gate = 0.f, up = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+      gate += ei::to_f32<TI>(g[s * split_stride]);
+      up += ei::to_f32<TI>(g[s * split_stride + I]);
+    }
+    const float act = gate / (1.0f + expf(-gate));
+    out[idx] = ei::from_f32<TO>(act * up);
+  }
+}
+
+}  // namespace
+
+extern "C" int ei_embed_gather(const int32_t* ids, const void* table, int table_dtype, float* out,
+                               int N, int H, int V, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && H > 0 && V > 0, "embed_gather: sizes must be positive");
+  EI_REQUIRE(ids && table && out, "embed_gather: null pointer");
+  const int threads = H >= 1024 ? 256 : 64;
+  if (table_dtype == EI_F32)
+    embed_gather_kernel<float><<<N, threads, 0, stream>>>(ids, static_cast<const float*>(table),
+                                                          out, H, V);
+  else if (table_dtype == EI_BF16)
+    embed_gather_kernel<bf16_t><<<N, threads, 0, stream>>>(ids, static_cast<const bf16_t*>(table),
+                                                           out, H, V);
+  else
+    EI_REQUIRE(false, "embed_gather: unknown table dtype");
+  EI_LAUNCH_CHECK();
+}
+
+template <typename TD, typename TO>
+static void launch_add_rmsnorm(float* residual, const void* delta, int nsplit, size_t split_stride,
+                               const int32_t* rows, const float* weight, float eps, void* out,
+                               int N, int H, int write_residual, hipStream_t stream) {
+  const int threads = H >= 2048 ? 256 : (H >= 256 ? 128 : 64);
+  const size_t lds = static_cast<size_t>(H) * sizeof(float);
+  if (delta)
+    add_rmsnorm_kernel<TD, TO, true><<<N, threads, lds, stream>>>(
+        residual, static_cast<const TD*>(delta), nsplit, split_stride, rows, weight, eps,
+        static_cast<TO*>(out), H, write_residual);
+  else
+    add_rmsnorm_kernel<TD, TO, false><<<N, threads, lds, stream>>>(
+        residual, nullptr, 0, 0, rows, weight, eps, static_cast<TO*>(out), H, 0);
+}
+
+// residual: float32 [*, H].  delta: [nsplit][*, H] of delta_dtype or null.  rows: null
+// (row r reads residual row r) or int32 [N] source rows (negative: padding).
+extern "C" int ei_add_rmsnorm(float* residual, const void* delta, int delta_dtype, int nsplit,
+                              long long split_stride, const int32_t* rows, const float* weight,
+                              float eps, void* out, int out_dtype, int N, int H,
+                              int write_residual, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && H > 0, "add_rmsnorm: sizes must be positive");
+  EI_REQUIRE(H <= 16384, "add_rmsnorm: width above 16384 is not supported");
+  EI_REQUIRE(residual && weight && out, "add_rmsnorm: null pointer");
+  EI_REQUIRE(!delta || nsplit >= 1, "add_rmsnorm: nsplit must be at least 1");
+  EI_REQUIRE(eps > 0.f, "add_rmsnorm: eps must be positive");
+  const size_t ss = static_cast<size_t>(split_stride);
+  if (delta_dtype == EI_F32 && out_dtype == EI_F32)
+    launch_add_rmsnorm<float, float>(residual, delta, nsplit, ss, rows, weight, eps, out, N, H,
+                                     write_residual, stream);
+  else if (delta_dtype == EI_F32 && out_dtype == EI_BF16)
+    launch_add_rmsnorm<float, bf16_t>(residual, delta, nsplit, ss, rows, weight, eps, out, N, H,
+                                      write_residual, stream);
+  else if (delta_dtype == EI_BF16 && out_dtype == EI_BF16)
+    launch_add_rmsnorm<bf16_t, bf16_t>(residual, delta, nsplit, ss, rows, weight, eps, out, N, H,
+                                       write_residual, stream);
+  else if (delta_dtype == EI_BF16 && out_dtype == EI_F32)
+    launch_add_rmsnorm<bf16_t, float>(residual, delta, nsplit, ss, rows, weight, eps, out, N, H,
+                                      write_residual, stream);
+  else
+    EI_REQUIRE(false, "add_rmsnorm: unknown dtype");
+  EI_LAUNCH_CHECK();
+}
+
+// gate_up: [nsplit][N, 2I] (gate columns first), out: [N, I].
+extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long long split_stride,
+                         void* out, int out_dtype, int N, int I, hipStream_t stream) {
+  EI_REQUIRE(N > 0 && I > 0 && nsplit >= 1, "swiglu: sizes must be positive");
+  EI_REQUIRE(gate_up && out, "swiglu: null pointer");
+  const size_t total = static_cast<size_t>(N) * I;
+  const int threads = 256;
+  size_t blocks = (total + threads - 1) / threads;
+  if (blocks > 256 * 32) blocks = 256 * 32;
+  const size_t ss = static_cast<size_t>(split_stride);
+  if (in_dtype == EI_F32 && out_dtype == EI_F32)
+    swiglu_kernel<float, float><<<blocks, threads, 0, stream>>>(
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total);
+  else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
+    swiglu_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>(
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total);
+  else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
+    swiglu_kernel<bf16_t, bf16_t><<<blocks, threads, 0, stream>>>(
+        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total);
+  else
+    EI_REQUIRE(false, "swiglu: unsupported dtype combination");
+  EI_LAUNCH_CHECK();
+}

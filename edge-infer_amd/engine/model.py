@@ -1,0 +1,145 @@
+"""The decoder model: embedding, the layers in schedule order, final norm, head.
+
+`DecoderModel` is built from a `ModelSpec` and a dictionary of parameters; it owns
+immutable weights on the device and nothing that changes between steps (sessions
+own caches and workspaces).  Its `forward` is the one step function: it runs the
+rows of a `StepContext` and returns float32 logits at the wanted rows.
+
+Order of operations: runtime/include/execution/decoder.hpp:109-171 and
+runtime/src/qwen3.cpp:293-299 of the reference (embedding, blocks, final norm,
+head); the head is applied to the wanted rows only.
+"""
+from __future__ import annotations
+
+from typing import Callable, Dict, Mapping, Tuple
+
+import torch
+
+from ..config.specs import ModelSpec
+from ..csrc import lib
+from ..parts.linear import Linear
+from ..parts.registry import lookup
+from ..weights.loader import ParamSpec
+
+DTYPES = {"float32": torch.float32, "fp32": torch.float32, "bfloat16": torch.bfloat16,
+          "bf16": torch.bfloat16, torch.float32: torch.float32, torch.bfloat16: torch.bfloat16}
+
+
+def resolve_dtype(dtype):
+    try:
+        return DTYPES[dtype]
+    except KeyError:
+        raise ValueError(f"dtype must be 'bfloat16' or 'float32', got {dtype!r}") from None
+
+
+def model_parameters(spec: ModelSpec) -> Dict[str, ParamSpec]:
+    """Every parameter of the model by its path."""
+    params = {"embed.weight": ParamSpec((spec.vocab_size, spec.hidden_size))}
+    for index, layer in enumerate(spec.layers):
+        block_cls = lookup("block", layer.block)
+        for name, param in block_cls.parameters(layer, spec.hidden_size).items():
+            params[f"layers.{index}.{name}"] = param
+    final_cls = lookup("norm", spec.final_norm.kind)
+    for name, param in final_cls.parameters(spec.final_norm, spec.hidden_size).items():
+        params[f"final_norm.{name}"] = param
+    params["head.weight"] = ParamSpec((spec.vocab_size, spec.hidden_size))
+    return params
+
+
+def expected_parameters(spec: ModelSpec, checkpoint_name: Callable[[str], str]
+                        ) -> Dict[str, Tuple[str, ParamSpec]]:
+    """parameter path -> (checkpoint tensor name, spec)."""
+    return {path: (checkpoint_name(path), param)
+            for path, param in model_parameters(spec).items()}
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, params: Mapping[str, torch.Tensor], dtype, device):
+        spec.validate()
+        self.spec = spec
+        self.dtype = resolve_dtype(dtype)
+        self.device = torch.device(device)
+        wanted = model_parameters(spec)
+        missing = [p for p in wanted if p not in params
+                   and not (p == "head.weight" and spec.tie_word_embeddings)]
+        if missing:
+            raise KeyError(f"model parameters missing: {missing}")
+        self._positions = {}
+        self.embed = params["embed.weight"].to(device=self.device, dtype=self.dtype).contiguous()
+        self.layers = []
+        for index, layer in enumerate(spec.layers):
+            prefix = f"layers.{index}."
+            own = {name[len(prefix):]: tensor for name, tensor in params.items()
+                   if name.startswith(prefix)}
+            block_cls = lookup("block", layer.block)
+            self.layers.append(block_cls(layer, spec.hidden_size, own, self.dtype, self.device,
+                                         positions=self.position_table))
+        final_cls = lookup("norm", spec.final_norm.kind)
+        self.final_norm = final_cls(spec.final_norm, spec.hidden_size,
+                                    {"weight": params["final_norm.weight"]}, self.dtype,
+                                    self.device)
+        if "head.weight" in params and params["head.weight"] is not params["embed.weight"]:
+            self.head = Linear(params["head.weight"], self.dtype, self.device)
+        else:  # tied: the head is the embedding table itself
+            self.head = Linear.__new__(Linear)
+            self.head.weight = self.embed
+            self.head.out_features, self.head.in_features = self.embed.shape
+            self.head.dtype = self.dtype
+
+    def position_table(self, position_spec):
+        """One shared encoding object per distinct position spec."""
+        table = self._positions.get(position_spec)
+        if table is None:
+            table = lookup("position", position_spec.kind)(position_spec, self.device)
+            self._positions[position_spec] = table
+        return table
+
+    def attention_item_sizes(self):
+        sizes = set()
+        for layer in self.layers:
+            mixer = getattr(layer, "mixer", None)
+            if mixer is not None and hasattr(mixer, "positions_per_item"):
+                sizes.add(mixer.positions_per_item())
+        return tuple(sorted(sizes))
+
+    def max_positions(self) -> int:
+        limit = self.spec.max_position_embeddings
+        for table in self._positions.values():
+            if table.max_positions is not None:
+                limit = min(limit, table.max_positions)
+        return limit
+
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+
+        def visit(obj):
+            nonlocal total
+            if isinstance(obj, torch.Tensor):
+                if obj.data_ptr() not in seen:
+                    seen.add(obj.data_ptr())
+                    total += obj.numel() * obj.element_size()
+            elif hasattr(obj, "__dict__"):
+                for value in vars(obj).values():
+                    visit(value)
+        visit(self.embed)
+        for layer in self.layers:
+            visit(layer)
+        visit(self.final_norm)
+        visit(self.head)
+        return total
+
+    # ------------------------------------------------------------------
+    def forward(self, ctx) -> torch.Tensor:
+        """Run the rows of `ctx`; float32 logits [wanted rows, vocab]."""
+        spec = self.spec
+        meta = ctx.meta
+        residual = ctx.buffer("residual", (ctx.n_rows, spec.hidden_size), torch.float32)
+        lib.embed_gather(meta.tokens, self.embed, residual)
+        pending = None
+        for entry in spec.schedule:
+            pending = self.layers[entry.layer].forward(ctx, residual, pending, entry)
+        if meta.n_want == 0:
+            return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
+        hidden = self.final_norm.add_norm(ctx, residual, pending, "final.h", rows=meta.want_rows,
+                                          write_residual=False)
+        return self.head.forward_f32(ctx, hidden, "logits")

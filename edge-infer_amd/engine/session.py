@@ -1,0 +1,127 @@
+"""A session: the mutable side of generation for one model.
+
+It owns the cache (slots, pages, fixed-size state), the workspaces and the metadata
+buffers, and offers the step function: `step(entries)` runs exactly the tokens it
+is given, as one batch, from what earlier steps left in the cache, and returns
+float32 logits at the wanted places.  Requests are validated before anything is
+written (token ids, live slots, room in the cache), so a refused step leaves the
+session as it was; the reference holds the same contract, runtime/src/qwen3.cpp:405-418.
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.allocator import PAGE_TOKENS, CacheFull
+from ..cache.storage import CacheLayout, SessionCache
+from ..parts.base import StepContext, Workspace
+from .batch import DeviceMeta, SeqStep, StepPlan
+
+
+class _Context(StepContext):
+    def __init__(self, session, **kwargs):
+        super().__init__(**kwargs)
+        self._session = session
+
+    def decode_splits(self, n_kv_heads: int) -> int:
+        """How many blocks share the key range of one (sequence, kv head) in decode:
+        enough to put about two blocks on each of the 256 compute units, never more
+        than there are pages."""
+        pages = max(1, (self.max_context + PAGE_TOKENS - 1) // PAGE_TOKENS)
+        wanted = (512 + self.n_seqs * n_kv_heads - 1) // (self.n_seqs * n_kv_heads)
+        return max(1, min(wanted, pages, 32))
+
+
+class Session:
+    def __init__(self, model, max_tokens: int, max_seqs: Optional[int] = None):
+        self.model = model
+        self.device = model.device
+        self.dtype = model.dtype
+        if max_tokens < 1:
+            raise ValueError("max_tokens must be positive")
+        n_pages = (max_tokens + PAGE_TOKENS - 1) // PAGE_TOKENS
+        if max_seqs is None:
+            max_seqs = min(n_pages, 256)
+        self.cache = SessionCache(CacheLayout(model.spec), max_tokens, max_seqs, self.dtype,
+                                  self.device, model.max_positions())
+        self.workspace = Workspace(self.device)
+        self.meta = DeviceMeta(self.device)
+        self._item_sizes = model.attention_item_sizes()
+        self.steps_run = 0
+
+    # -- slots -----------------------------------------------------------
+    def begin(self) -> int:
+        """Take a slot for a new sequence (length 0)."""
+        return self.cache.acquire()
+
+    def end(self, slot: int) -> None:
+        """Give a slot and everything it holds back."""
+        self.cache.release(slot)
+
+    def reset(self) -> None:
+        """End every live sequence; allocations are kept."""
+        torch.cuda.synchronize(self.device)
+        self.cache.release_all()
+
+    def length(self, slot: int) -> int:
+        if not self.cache.slots.is_live(slot):
+            raise ValueError(f"slot {slot} is not live")
+        return self.cache.lengths[slot]
+
+    @property
+    def capacity(self) -> int:
+        """Most tokens one sequence can hold."""
+        return self.cache.max_seq_tokens
+
+    # -- the step function -------------------------------------------------
+    def _validate(self, entries) -> List[SeqStep]:
+        vocab = self.model.spec.vocab_size
+        seqs: List[SeqStep] = []
+        seen = set()
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        for slot, tokens, want in entries:
+            if not self.cache.slots.is_live(slot):
+                raise ValueError(f"slot {slot} is not live")
+            if slot in seen:
+                raise ValueError(f"slot {slot} appears twice in one step")
+            seen.add(slot)
+            tokens = list(tokens)
+            if not tokens:
+                raise ValueError("an entry brings at least one token")
+            for token in tokens:
+                if not isinstance(token, int) or isinstance(token, bool) \
+                        or not 0 <= token < vocab:
+                    raise ValueError(f"token id {token!r} is outside the vocabulary of {vocab}")
+            want = list(want)
+            for w in want:
+                if not 0 <= w < len(tokens):
+                    raise ValueError(f"wanted place {w} is outside the {len(tokens)} tokens given")
+            seqs.append(SeqStep(slot=slot, start=self.cache.lengths[slot], tokens=tokens,
+                                want=want))
+        return seqs
+
+    def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> torch.Tensor:
+        """entries: (slot, next tokens, wanted places among them).  Returns float32
+        logits [number of wanted places, vocab] in the order of entries and places."""
+        seqs = self._validate(entries)
+        growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
+        self.cache.check_growth(growth)          # raises before anything changes
+        self.cache.grow(growth)
+        plan = StepPlan(seqs, item_sizes=self._item_sizes)
+        logits = self._run(plan, self.meta, self.workspace)
+        self.cache.commit(growth)
+        self.steps_run += 1
+        return logits
+
+    def _run(self, plan: StepPlan, meta: DeviceMeta, workspace: Workspace) -> torch.Tensor:
+        slots = [seq.slot for seq in plan.seqs]
+        tables = [self.cache.page_rows(group, slots, plan.n_seqs)
+                  for group in range(len(self.cache.kv_pages))]
+        meta.upload(plan, tables)
+        ctx = _Context(self, dtype=self.dtype, device=self.device, n_rows=plan.n_rows,
+                       n_seqs=plan.n_seqs, decode=plan.decode, meta=meta, cache=self.cache,
+                       workspace=workspace, max_context=plan.max_context)
+        ctx.sequences = plan.seqs
+        return self.model.forward(ctx)

@@ -1,0 +1,101 @@
+"""Causal grouped-query attention over the paged key/value cache.
+
+x -> fused q/k/v projection -> (optional) per-head RMSNorm of q and k -> rotary
+encoding -> keys and values stored in the cache -> attention over the cache ->
+output projection.  The order follows the reference's decoder,
+runtime/include/execution/decoder.hpp:121-158.  Three separate checkpoint matrices
+become one [Q + 2 KV, H] matrix when the part is built: each output element is
+still the same dot product.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..csrc import lib
+from ..weights.loader import ParamSpec
+from .base import KVRequest
+from .linear import Linear
+from .registry import lookup
+
+
+class Attention:
+    @classmethod
+    def parameters(cls, spec, hidden):
+        params = {
+            "q_proj.weight": ParamSpec((spec.q_width, hidden)),
+            "k_proj.weight": ParamSpec((spec.kv_width, hidden)),
+            "v_proj.weight": ParamSpec((spec.kv_width, hidden)),
+            "o_proj.weight": ParamSpec((hidden, spec.q_width)),
+        }
+        if spec.qk_norm:
+            params["q_norm.weight"] = ParamSpec((spec.head_dim,), init="norm")
+            params["k_norm.weight"] = ParamSpec((spec.head_dim,), init="norm")
+        return params
+
+    @classmethod
+    def cache_request(cls, spec):
+        return KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window)
+
+    @classmethod
+    def check(cls, spec):
+        if spec.n_heads % spec.n_kv_heads:
+            raise ValueError("attention: n_heads must be a multiple of n_kv_heads")
+        if spec.head_dim % 16 or not 16 <= spec.head_dim <= 256:
+            raise ValueError("attention: head_dim must be a multiple of 16 between 16 and 256, "
+                             f"got {spec.head_dim}")
+        if spec.window is not None and spec.window < 1:
+            raise ValueError("attention: a window must be at least 1")
+
+    def __init__(self, spec, hidden, params, dtype, device, positions):
+        self.check(spec)
+        self.spec = spec
+        self.hidden = hidden
+        self.dtype = dtype
+        fused = torch.cat([params["q_proj.weight"], params["k_proj.weight"],
+                           params["v_proj.weight"]], dim=0)
+        self.qkv = Linear(fused, dtype, device)
+        self.o = Linear(params["o_proj.weight"], dtype, device)
+        self.q_norm = self.k_norm = None
+        if spec.qk_norm:
+            self.q_norm = params["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+            self.k_norm = params["k_norm.weight"].to(device=device, dtype=torch.float32).contiguous()
+        self.position = positions(spec.position)   # shared table object
+        self.group = spec.n_heads // spec.n_kv_heads
+        self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
+
+    # the number of positions of one sequence that a prefill work item covers
+    def positions_per_item(self):
+        return lib.attention_positions_per_item(self.group)
+
+    def forward(self, ctx, x, entry):
+        spec = self.spec
+        n = x.shape[0]
+        meta = ctx.meta
+        group_index, k_pages, v_pages = ctx.cache.kv(entry.cache)
+        page_table = meta.page_table(group_index)
+        qkv = self.qkv.forward(ctx, x, "attn.qkv")
+        q = ctx.buffer("attn.q", (n, spec.q_width))
+        lib.qk_norm_rope_store(
+            qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, self.position.table, meta.row_pos,
+            meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads, spec.n_kv_heads,
+            spec.head_dim, write_cache=entry.writes_cache)
+        out = ctx.buffer("attn.out", (n, spec.q_width))
+        if ctx.decode:
+            splits = ctx.decode_splits(spec.n_kv_heads)
+            part_o = part_ml = None
+            if splits > 1:
+                part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
+                                    torch.float32)
+                part_ml = ctx.buffer("attn.part_ml", (n * spec.n_heads * splits * 2,),
+                                     torch.float32)
+            item_seq, item_row0, item_npos, n_items = meta.decode_items()
+            lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                          meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                          spec.n_kv_heads, spec.head_dim, window=spec.window, scale=self.scale,
+                          n_splits=splits, part_o=part_o, part_ml=part_ml)
+        else:
+            item_seq, item_row0, item_npos, n_items = meta.prefill_items(self.positions_per_item())
+            lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                          meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                          spec.n_kv_heads, spec.head_dim, window=spec.window, scale=self.scale)
+        return self.o.forward(ctx, out, "attn.o")

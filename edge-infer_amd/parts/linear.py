@@ -1,0 +1,59 @@
+"""y = x . W^T for a checkpoint matrix kept in its stored [out, in] layout.
+
+float32: the hand-written float32 kernel (no reduced-precision matrix mode).
+bfloat16: for up to `SKINNY_ROWS` rows the hand-written weight-streaming MFMA
+kernel, which returns float32 partial sums [splits, rows, out] that the consuming
+kernel adds up; for more rows the library matrix product (the reference multiplies
+through cuBLAS as well, operators/src/cuda/execution.cu:299-324).
+"""
+from __future__ import annotations
+
+import torch
+
+from ..csrc import lib
+
+SKINNY_ROWS = 64
+
+
+class Linear:
+    def __init__(self, weight: torch.Tensor, dtype, device):
+        if weight.dim() != 2:
+            raise ValueError("a linear weight must be a matrix [out, in]")
+        self.weight = weight.to(device=device, dtype=dtype).contiguous()
+        self.out_features, self.in_features = self.weight.shape
+        self.dtype = dtype
+
+    def forward(self, ctx, x: torch.Tensor, out_name: str) -> torch.Tensor:
+        """x [N, in] of the step's storage type -> [N, out] (or float32 partial sums
+        [splits, N, out]); the result lives in the workspace buffer `out_name`."""
+        rows = x.shape[0]
+        if self.dtype == torch.float32:
+            out = ctx.buffer(out_name, (rows, self.out_features), torch.float32)
+            lib.gemm_f32(x, self.weight, out)
+            return out
+        if rows <= SKINNY_ROWS and lib.has_skinny_gemm():
+            splits = lib.skinny_gemm_splits(rows, self.out_features, self.in_features)
+            out = ctx.buffer(out_name + ".f32", (splits, rows, self.out_features), torch.float32)
+            lib.gemm_bf16_skinny(x, self.weight, out)
+            return out
+        out = ctx.buffer(out_name, (rows, self.out_features), torch.bfloat16)
+        torch.matmul(x, self.weight.t(), out=out)
+        return out
+
+    def forward_f32(self, ctx, x: torch.Tensor, out_name: str) -> torch.Tensor:
+        """Like forward, but one float32 [N, out] tensor (used for the logits)."""
+        rows = x.shape[0]
+        out = ctx.buffer(out_name, (rows, self.out_features), torch.float32)
+        if self.dtype == torch.float32:
+            lib.gemm_f32(x, self.weight, out)
+            return out
+        if lib.has_skinny_gemm():
+            for start in range(0, rows, SKINNY_ROWS):
+                stop = min(rows, start + SKINNY_ROWS)
+                lib.gemm_bf16_skinny(x[start:stop], self.weight, out[start:stop].unsqueeze(0),
+                                     splits=1)
+            return out
+        low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)
+        torch.matmul(x, self.weight.t(), out=low)
+        out.copy_(low)
+        return out
