@@ -1,0 +1,99 @@
+"""Python entry point in the manner of the reference's `model_bridge`
+(bindings/python/model_bridge.cpp:245-294, docs/python-api.md):
+
+    config, weights, model_type = load_checkpoint(path, "qwen3_bf16")
+    model = Model(config, weights, model_type, device="cuda")
+    session = model.new_session(capacity=1024)
+    session.generate(prompt_ids, tokens.append, max_length=len(prompt_ids) + 32, top_k=1)
+    session.reset()
+
+`Model` prepares weights and holds no cache; sessions share its weights and own
+their caches.  Beyond the reference, a session can serve a batch of prompts
+(`new_session(max_batch=8)`, `session.generate_batch`) and exposes the step function
+(`session.step`).  Model types: "qwen3_bf16" (the reference's name) and
+"qwen3_fp32" for the true 32-bit path.
+"""
+from __future__ import annotations
+
+import json
+from pathlib import Path
+from typing import Mapping, Optional
+
+import torch
+
+from . import require_gpu
+from .config import read_config, resolve_architecture
+from .engine.generate import generate  # noqa: F401  (re-exported)
+from .engine.model import DecoderModel, expected_parameters
+from .engine.session import Session
+from .sampling.params import SamplingParams  # noqa: F401
+from .weights import match_parameters, read_tensors
+
+MODEL_TYPES = {"qwen3_bf16": "bfloat16", "qwen3_fp32": "float32"}
+DEFAULT_CAPACITY = 4096   # bindings/python/model_bridge.cpp:135-141: min(4096, model limit)
+
+
+def load_checkpoint(model_path, model_type="qwen3_bf16"):
+    """(config dict, {tensor name: tensor}, model type) of a local folder; nothing is
+    ever downloaded (frontend/checkpoint.py:58-105)."""
+    if model_type not in MODEL_TYPES:
+        raise ValueError(f"unsupported model type '{model_type}'; known: {sorted(MODEL_TYPES)}")
+    root = Path(model_path).resolve()
+    with (root / "config.json").open(encoding="utf-8") as source:
+        config = json.load(source)
+    if not isinstance(config, dict):
+        raise ValueError("config.json must hold a JSON object")
+    return config, read_tensors(root), model_type
+
+
+class Model:
+    def __init__(self, config: Mapping, weights: Mapping[str, torch.Tensor],
+                 model_type: str = "qwen3_bf16", device: Optional[str] = None):
+        if model_type not in MODEL_TYPES:
+            raise ValueError(f"unsupported model type '{model_type}'; known: {sorted(MODEL_TYPES)}")
+        if device not in (None, "cuda") and not str(device).startswith("cuda"):
+            raise ValueError("this library runs on the GPU only (device 'cuda')")
+        self._device = require_gpu(device or "cuda")
+        entry = resolve_architecture(config)
+        self.config = entry.config_class.from_dict(config)
+        spec = self.config.model_spec()
+        expected = expected_parameters(spec, self.config.checkpoint_name)
+        optional = {"head.weight": "embed.weight"} if spec.tie_word_embeddings else {}
+        params = match_parameters(expected, weights, optional=optional,
+                                  aliases=getattr(self.config, "checkpoint_aliases", {}))
+        factory = entry.model_factory or DecoderModel
+        self.decoder = factory(spec, params, MODEL_TYPES[model_type], self._device)
+        self.decoder.config = self.config
+        self.model_type = model_type
+
+    @classmethod
+    def from_pretrained(cls, model_path, model_type="qwen3_bf16", device=None) -> "Model":
+        config, weights, model_type = load_checkpoint(model_path, model_type)
+        return cls(config, weights, model_type, device)
+
+    @property
+    def device(self) -> str:
+        return str(self._device)
+
+    @property
+    def max_context_length(self) -> int:
+        return self.decoder.max_positions()
+
+    def new_session(self, capacity: Optional[int] = None, max_batch: int = 1,
+                    seed: int = 0) -> Session:
+        """An independent session whose sequences hold up to `capacity` tokens each
+        (default min(4096, model limit)), `max_batch` of them at a time."""
+        limit = self.max_context_length
+        if capacity is None:
+            capacity = min(DEFAULT_CAPACITY, limit)
+        if isinstance(capacity, bool) or not isinstance(capacity, int) or not 1 <= capacity <= limit:
+            raise ValueError(f"capacity must lie in 1..{limit}, got {capacity!r}")
+        if max_batch < 1:
+            raise ValueError("max_batch must be positive")
+        pages_each = (capacity + 63) // 64
+        return Session(self.decoder, max_tokens=pages_each * 64 * max_batch, max_seqs=max_batch,
+                       max_seq_tokens=capacity, seed=seed)
+
+
+def is_gpu_available() -> bool:
+    return torch.cuda.is_available()

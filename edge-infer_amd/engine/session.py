@@ -34,7 +34,8 @@ class _Context(StepContext):
 
 
 class Session:
-    def __init__(self, model, max_tokens: int, max_seqs: Optional[int] = None):
+    def __init__(self, model, max_tokens: int, max_seqs: Optional[int] = None,
+                 max_seq_tokens: Optional[int] = None, seed: int = 0):
         self.model = model
         self.device = model.device
         self.dtype = model.dtype
@@ -43,8 +44,16 @@ class Session:
         n_pages = (max_tokens + PAGE_TOKENS - 1) // PAGE_TOKENS
         if max_seqs is None:
             max_seqs = min(n_pages, 256)
+        limit = model.max_positions()
+        if max_seq_tokens is not None:
+            if not 1 <= max_seq_tokens <= limit:
+                raise ValueError(f"a sequence capacity must lie in 1..{limit}, got {max_seq_tokens}")
+            limit = max_seq_tokens
         self.cache = SessionCache(CacheLayout(model.spec), max_tokens, max_seqs, self.dtype,
-                                  self.device, model.max_positions())
+                                  self.device, limit)
+        self.seed = int(seed)
+        self._streams_used = 0
+        self._sampler = None
         self.workspace = Workspace(self.device)
         self.meta = DeviceMeta(self.device)
         self._item_sizes = model.attention_item_sizes()
@@ -73,6 +82,51 @@ class Session:
     def capacity(self) -> int:
         """Most tokens one sequence can hold."""
         return self.cache.max_seq_tokens
+
+    @property
+    def max_batch(self) -> int:
+        return self.cache.n_slots
+
+    def free_tokens(self) -> int:
+        if not self.cache.kv_pools:
+            return self.cache.n_pages * PAGE_TOKENS
+        return min(pool.n_free for pool in self.cache.kv_pools) * PAGE_TOKENS
+
+    # -- generation ----------------------------------------------------------
+    def generate_batch(self, prompts, *, max_length=None, max_new_tokens=None, temperature=1.0,
+                       top_p=0.9, top_k=1, seed=None, stop_ids=None, callback=None,
+                       max_batch=None, first_stream=None):
+        """New tokens for every prompt (lists of ints), served in batches of prompts
+        that start together.  `callback(index, token)` sees each delivered token."""
+        from ..sampling.params import SamplingParams
+        from ..sampling.sampler import Sampler
+        from .generate import generate
+        if self._sampler is None:
+            self._sampler = Sampler(self.device)
+        spec = self.model.spec
+        if stop_ids is None:
+            stop_ids = (spec.eos_token_id,)
+        if first_stream is None:
+            first_stream = self._streams_used
+            self._streams_used += len(prompts)
+        params = SamplingParams(temperature=float(temperature), top_p=float(top_p),
+                                top_k=int(top_k), seed=self.seed if seed is None else int(seed))
+        return generate(self, self._sampler, prompts, vocab_size=spec.vocab_size,
+                        max_length=max_length, max_new_tokens=max_new_tokens, params=params,
+                        stop_ids=stop_ids, callback=callback, max_batch=max_batch,
+                        first_stream=first_stream)
+
+    def generate(self, input_ids, callback=None, max_length=100, temperature=1.0, top_p=0.9,
+                 top_k=1, seed=None):
+        """One complete fresh prompt; `max_length` counts prompt plus generated tokens;
+        `callback(token)` sees every delivered token; the end-of-sequence token ends
+        the request and is not delivered.  Names, meanings and defaults of the
+        reference's Session.generate (bindings/python/model_bridge.cpp:248-252).
+        Returns the delivered tokens."""
+        wrapped = None if callback is None else (lambda index, token: callback(token))
+        return self.generate_batch([list(input_ids)], max_length=max_length,
+                                   temperature=temperature, top_p=top_p, top_k=top_k, seed=seed,
+                                   callback=wrapped)[0]
 
     # -- the step function -------------------------------------------------
     def _validate(self, entries) -> List[SeqStep]:

@@ -1,0 +1,69 @@
+"""Shared test fixtures: two tiny Qwen3 configurations that differ in every size and
+option, and tolerances that are fixed here once."""
+import json
+import tempfile
+from pathlib import Path
+
+import torch
+
+# float32 engine against the float64 plain implementation, relative to the largest logit
+F32_REL = 1e-4
+# bfloat16 engine against the plain implementation: root-mean-square and maximum error
+# relative to the root-mean-square and the maximum logit (bfloat16 keeps 8 significant
+# bits, 2^-9 relative per rounding; a few dozen roundings accumulate per token)
+BF16_RMS_REL = 2e-2
+BF16_MAX_REL = 6e-2
+
+TINY_A = dict(vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
+              num_key_value_heads=2, head_dim=16, intermediate_size=128,
+              max_position_embeddings=128, bos_token_id=0, eos_token_id=255, rms_norm_eps=1e-6,
+              rope_theta=10000.0, tie_word_embeddings=True)
+TINY_B = dict(vocab_size=381, hidden_size=96, num_hidden_layers=3, num_attention_heads=8,
+              num_key_value_heads=1, head_dim=32, intermediate_size=200,
+              max_position_embeddings=256, bos_token_id=1, eos_token_id=380, rms_norm_eps=1e-5,
+              rope_theta=1000000.0, tie_word_embeddings=False)
+SEEDS = {"A": 0, "B": 1}
+CONFIGS = {"A": TINY_A, "B": TINY_B}
+
+
+def tiny_config(name):
+    from edge_infer_amd import Qwen3Config
+    return Qwen3Config(**CONFIGS[name])
+
+
+def make_folder(name, root):
+    from edge_infer_amd import write_model_folder
+    path = Path(root) / f"tiny_{name}"
+    if not (path / "model.safetensors").is_file():
+        write_model_folder(path, tiny_config(name), SEEDS[name])
+    return path
+
+
+def random_ids(vocab, count, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (count,), generator=g).tolist()
+
+
+def assert_close_f32(actual, expected, what=""):
+    actual, expected = actual.double().cpu(), expected.double().cpu()
+    scale = expected.abs().max().item()
+    err = (actual - expected).abs().max().item()
+    assert err <= F32_REL * scale, f"{what}: max error {err:.3e} against scale {scale:.3e}"
+
+
+def assert_close_bf16(actual, expected, what=""):
+    actual, expected = actual.double().cpu(), expected.double().cpu()
+    diff = actual - expected
+    rms = diff.pow(2).mean().sqrt().item()
+    ref_rms = expected.pow(2).mean().sqrt().item()
+    worst = diff.abs().max().item()
+    scale = expected.abs().max().item()
+    assert rms <= BF16_RMS_REL * ref_rms, f"{what}: rms error {rms:.3e} against {ref_rms:.3e}"
+    assert worst <= BF16_MAX_REL * scale, f"{what}: max error {worst:.3e} against {scale:.3e}"
+
+
+def assert_close(dtype, actual, expected, what=""):
+    if dtype == "float32":
+        assert_close_f32(actual, expected, what)
+    else:
+        assert_close_bf16(actual, expected, what)

@@ -1,0 +1,121 @@
+"""Loading by tensor name, precision kept, one error for everything wrong (no GPU)."""
+import json
+
+import pytest
+import torch
+from safetensors.torch import load_file, save_file
+
+from edge_infer_amd import Qwen3Config, WeightsError, write_model_folder
+from edge_infer_amd.engine.model import expected_parameters, model_parameters
+from edge_infer_amd.weights import match_parameters, read_tensors
+from helpers import make_folder, tiny_config
+
+
+def expected_for(name):
+    cfg = tiny_config(name)
+    return cfg, expected_parameters(cfg.model_spec(), cfg.checkpoint_name)
+
+
+def test_random_folder_round_trip(tmp_path):
+    folder = make_folder("B", tmp_path)
+    cfg, expected = expected_for("B")
+    assert Qwen3Config.from_dict(json.loads((folder / "config.json").read_text())) == cfg
+    tensors = read_tensors(folder)
+    params = match_parameters(expected, tensors)
+    assert set(params) == set(expected)
+    assert all(t.dtype == torch.bfloat16 for t in tensors.values())
+    q = params["layers.2.mixer.q_proj.weight"]
+    assert tuple(q.shape) == (8 * 32, 96)                 # [out, in] as stored
+    assert abs(q.float().std().item() - 0.02) < 0.002     # N(0, 0.02)
+    n = params["layers.0.norm1.weight"].float()
+    assert 0.9 <= n.min() and n.max() <= 1.1 and n.std() > 0.03   # 1 + U(-0.1, 0.1)
+    # the same seed gives the same bytes, another seed does not
+    again = write_model_folder(tmp_path / "again", cfg, 1)
+    other = write_model_folder(tmp_path / "other", cfg, 2)
+    a, b, c = (load_file(str(p / "model.safetensors")) for p in (folder, again, other))
+    assert all(torch.equal(a[k], b[k]) for k in a)
+    assert not torch.equal(a["lm_head.weight"], c["lm_head.weight"])
+
+
+def test_tied_head_is_not_stored_and_resolves_to_the_embedding(tmp_path):
+    folder = make_folder("A", tmp_path)
+    cfg, expected = expected_for("A")
+    tensors = read_tensors(folder)
+    assert "lm_head.weight" not in tensors
+    params = match_parameters(expected, tensors, optional={"head.weight": "embed.weight"})
+    assert params["head.weight"] is params["embed.weight"]
+    # untied configuration without a head: one clear error
+    with pytest.raises(WeightsError, match="lm_head.weight"):
+        match_parameters(expected, tensors)
+    # an explicit head wins over the tie, also under its alias
+    tensors["model.lm_head.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)
+    params = match_parameters(expected, tensors, optional={"head.weight": "embed.weight"},
+                              aliases=cfg.checkpoint_aliases)
+    assert params["head.weight"] is tensors["model.lm_head.weight"]
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    folder = make_folder("B", tmp_path)
+    _, expected = expected_for("B")
+    tensors = read_tensors(folder)
+    del tensors["model.layers.1.mlp.up_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.7.self_attn.q_proj.weight"] = torch.zeros(2, 2)
+    tensors["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(256)
+    tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(96, 32)   # transposed
+    with pytest.raises(WeightsError) as info:
+        match_parameters(expected, tensors)
+    error = info.value
+    assert sorted(error.missing) == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
+    assert error.unexpected == ["model.layers.0.self_attn.q_proj.bias",
+                                "model.layers.7.self_attn.q_proj.weight"]
+    assert error.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (32, 96), (96, 32))]
+    text = str(error)
+    for piece in ("missing tensors (2)", "unexpected tensors (2)", "wrong shapes (1)",
+                  "expected [32, 96] got [96, 32]"):
+        assert piece in text
+
+
+def test_stored_precision_is_kept(tmp_path):
+    tensors = {
+        "a": torch.randn(4, 4, dtype=torch.float32),
+        "b": torch.randn(4, 4).to(torch.bfloat16),
+        "c": torch.randn(4, 4).to(torch.float16),
+        "d": torch.arange(6, dtype=torch.int64),
+        "e": torch.randn(3, dtype=torch.float64),
+    }
+    (tmp_path / "config.json").write_text("{}")
+    save_file(tensors, str(tmp_path / "model.safetensors"))
+    loaded = read_tensors(tmp_path)
+    assert loaded["a"].dtype == torch.float32 and torch.equal(loaded["a"], tensors["a"])
+    assert loaded["b"].dtype == torch.bfloat16
+    assert loaded["c"].dtype == torch.bfloat16
+    assert loaded["d"].dtype == torch.int32 and loaded["d"].tolist() == list(range(6))
+    assert loaded["e"].dtype == torch.float32
+
+
+def test_sharded_checkpoint_and_path_containment(tmp_path):
+    save_file({"x": torch.ones(2)}, str(tmp_path / "part1.safetensors"))
+    save_file({"y": torch.zeros(3)}, str(tmp_path / "part2.safetensors"))
+    index = {"weight_map": {"x": "part1.safetensors", "y": "part2.safetensors"}}
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    loaded = read_tensors(tmp_path)
+    assert set(loaded) == {"x", "y"}
+    index["weight_map"]["y"] = "../outside.safetensors"
+    (tmp_path / "model.safetensors.index.json").write_text(json.dumps(index))
+    with pytest.raises(ValueError, match="inside"):
+        read_tensors(tmp_path)
+    (tmp_path / "model.safetensors.index.json").unlink()
+    with pytest.raises(FileNotFoundError):
+        read_tensors(tmp_path)
+
+
+def test_parameter_inventory_matches_the_architecture():
+    cfg = tiny_config("B")
+    params = model_parameters(cfg.model_spec())
+    per_layer = 11   # 2 norms, q k v o, q_norm k_norm, gate up down
+    assert len(params) == 3 + per_layer * cfg.num_hidden_layers
+    total = sum(torch.Size(p.shape).numel() for p in params.values())
+    H, V, I, Q, KV, d = 96, 381, 200, 256, 32, 32
+    layer = 2 * H + Q * H + 2 * KV * H + H * Q + 2 * d + 3 * I * H
+    assert total == 2 * V * H + H + 3 * layer
