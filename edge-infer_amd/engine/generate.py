@@ -132,7 +132,7 @@ def _run_batch(session, sampler, batch, params, stop, vocab_size, callback, all_
     try:
         for request in batch:
             request.slot = session.begin()
-        logits = session.step([(r.slot, r.prompt, [len(r.prompt) - 1]) for r in batch])
+        logits = session.step([(r.slot, r.prompt, [len(r.prompt) - 1]) for r in batch], copy=False)
         active = list(batch)
         while True:
             tokens = sampler(logits, params, [r.stream for r in active],
@@ -143,7 +143,7 @@ def _run_batch(session, sampler, batch, params, stop, vocab_size, callback, all_
             if not feed:
                 break
             active = [r for r, _ in feed]
-            logits = session.step([(r.slot, [token], [0]) for r, token in feed])
+            logits = session.step([(r.slot, [token], [0]) for r, token in feed], copy=False)
     finally:
         for request in batch:
             if request.slot >= 0:

@@ -156,9 +156,12 @@ class Session:
                                 want=want))
         return seqs
 
-    def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]]) -> torch.Tensor:
+    def step(self, entries: Sequence[Tuple[int, Sequence[int], Sequence[int]]],
+             copy: bool = True) -> torch.Tensor:
         """entries: (slot, next tokens, wanted places among them).  Returns float32
-        logits [number of wanted places, vocab] in the order of entries and places."""
+        logits [number of wanted places, vocab] in the order of entries and places.
+        With copy=False the result is a view of the session's workspace that the next
+        step overwrites."""
         seqs = self._validate(entries)
         growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
         self.cache.check_growth(growth)          # raises before anything changes
@@ -167,7 +170,7 @@ class Session:
         logits = self._run(plan, self.meta, self.workspace)
         self.cache.commit(growth)
         self.steps_run += 1
-        return logits
+        return logits.clone() if copy else logits
 
     def _run(self, plan: StepPlan, meta: DeviceMeta, workspace: Workspace) -> torch.Tensor:
         slots = [seq.slot for seq in plan.seqs]

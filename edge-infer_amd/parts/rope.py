@@ -17,9 +17,8 @@ class RotaryTable:
             raise ValueError("rotary dimension must be even")
         self.spec = spec
         half = spec.dim // 2
-        exponent = (2.0 * torch.arange(half, dtype=torch.float64)) / spec.dim
-        frequency = (1.0 / torch.pow(torch.tensor(float(spec.theta), dtype=torch.float64),
-                                     exponent)).to(torch.float32)
+        exponent = (2.0 * torch.arange(half, dtype=torch.float32)) / float(spec.dim)
+        frequency = 1.0 / torch.pow(torch.tensor(float(spec.theta), dtype=torch.float32), exponent)
         position = torch.arange(spec.max_positions, dtype=torch.float32)
         angle = (position[:, None] * frequency[None, :]).to(torch.float64)
         table = torch.cat([torch.cos(angle), torch.sin(angle)], dim=1).to(torch.float32)

@@ -37,7 +37,7 @@ class ScriptedSession:
         self.ended.append(slot)
         del self.live[slot]            # KeyError on a double release
 
-    def step(self, entries):
+    def step(self, entries, copy=True):
         self.steps.append([(slot, list(tokens), list(want)) for slot, tokens, want in entries])
         rows = []
         for slot, tokens, want in entries:
@@ -135,7 +135,7 @@ def test_invalid_requests_are_refused_before_anything_runs():
 
 def test_slots_are_returned_when_a_step_fails():
     class Failing(ScriptedSession):
-        def step(self, entries):
+        def step(self, entries, copy=True):
             if len(self.steps) == 1:
                 raise RuntimeError("boom")
             return super().step(entries)

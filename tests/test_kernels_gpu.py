@@ -1,0 +1,436 @@
+"""Each HIP kernel alone against its plain float64 reference, at sizes other than
+the engine's tiny models (odd widths, head sizes 16..256, group ratios 1..20)."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import plain_qwen3 as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda"
+PAGE = 64
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from edge_infer_amd.csrc import lib as kernels
+    return kernels
+
+
+def tol(dtype):
+    return 2e-6 if dtype == torch.float32 else 1.2e-2   # bfloat16: 2^-8 relative, some slack
+
+
+def close(actual, expected, dtype, scale=None):
+    actual, expected = actual.double().cpu(), expected.double().cpu()
+    scale = expected.abs().max().item() if scale is None else scale
+    err = (actual - expected).abs().max().item()
+    assert err <= tol(dtype) * max(scale, 1e-30), f"max error {err:.3e}, scale {scale:.3e}"
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_gather(lib, dtype):
+    V, H = 381, 200
+    table = torch.randn(V, H, device=DEV).to(dtype)
+    ids = torch.tensor([0, 380, 17, 17, 200], dtype=torch.int32, device=DEV)
+    out = torch.full((5, H), float("nan"), device=DEV)
+    lib.embed_gather(ids, table, out)
+    assert torch.equal(out.cpu(), plain.embedding(ids.cpu().tolist(), table.cpu()).float())
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H", [200, 4096 + 24])
+def test_add_rmsnorm(lib, out_dtype, H):
+    N, eps = 7, 1e-5
+    residual = torch.randn(N, H, device=DEV)
+    weight = (1 + 0.1 * torch.randn(H, device=DEV))
+    # no delta
+    out = torch.empty(N, H, device=DEV, dtype=out_dtype)
+    lib.add_rmsnorm(residual, None, weight, eps, out)
+    close(out, plain.rms_norm(residual.cpu(), weight.cpu(), eps), out_dtype)
+    # float32 delta in three splits: residual is updated, the norm sees the sum
+    delta = torch.randn(3, N, H, device=DEV)
+    before = residual.clone()
+    lib.add_rmsnorm(residual, delta, weight, eps, out)
+    total = before.double().cpu() + delta.double().cpu().sum(0)
+    close(residual, total, torch.float32)
+    close(out, plain.rms_norm(total, weight.cpu(), eps), out_dtype)
+    # bfloat16 delta
+    if out_dtype == torch.bfloat16:
+        d16 = torch.randn(N, H, device=DEV).to(torch.bfloat16)
+        before = residual.clone()
+        lib.add_rmsnorm(residual, d16, weight, eps, out)
+        close(residual, before.double().cpu() + d16.double().cpu(), torch.float32)
+    # gathered rows, one of them padding; the residual is left alone
+    rows = torch.tensor([4, -1, 0], dtype=torch.int32, device=DEV)
+    before = residual.clone()
+    delta2 = torch.randn(1, N, H, device=DEV)
+    out3 = torch.full((3, H), 7.0, device=DEV, dtype=out_dtype)
+    lib.add_rmsnorm(residual, delta2, weight, eps, out3, rows=rows, write_residual=False)
+    assert torch.equal(residual, before)
+    expect = plain.rms_norm(before.double().cpu() + delta2[0].double().cpu(), weight.cpu(), eps)
+    close(out3[0], expect[4], out_dtype)
+    close(out3[2], expect[0], out_dtype)
+    assert (out3[1] == 0).all()
+
+
+def test_rms_norm_reference_vector_on_the_gpu(lib):
+    """operators/tests/operators_cuda_bf16_contract_test.cu:235-284, float32 part (2e-6)."""
+    n = 128
+    x = torch.tensor([-0.8 + (i % 7) * 0.25 for i in range(n)], device=DEV).reshape(1, n)
+    w = torch.tensor([0.63 + (i % 5) * 0.17 for i in range(n)], device=DEV)
+    out = torch.empty(1, n, device=DEV)
+    lib.add_rmsnorm(x, None, w, 1e-6, out)
+    inv = 1.0 / math.sqrt(float((x.double() ** 2).sum()) / n + 1e-6)
+    assert (out.double() - x.double() * inv * w.double()).abs().max().item() < 2e-6
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu(lib, dtype):
+    N, I = 5, 200
+    gate_up = torch.randn(2, N, 2 * I, device=DEV) * 3
+    gate_up[0, 0, 0], gate_up[1, 0, 0] = -60.0, -28.0      # the reference's -88 tail case
+    out = torch.empty(N, I, device=DEV, dtype=dtype)
+    lib.swiglu(gate_up, out)
+    total = gate_up.double().cpu().sum(0)
+    close(out, plain.swiglu(total[:, :I], total[:, I:]), dtype)
+    assert torch.isfinite(out.float()).all()
+    if dtype == torch.bfloat16:
+        one = gate_up[0].to(dtype).contiguous()
+        lib.swiglu(one, out)
+        close(out, plain.swiglu(one.double().cpu()[:, :I], one.double().cpu()[:, I:]), dtype)
+
+
+@pytest.mark.parametrize("shape", [(1, 381, 96), (5, 64, 200), (70, 130, 33), (130, 257, 512)])
+def test_gemm_f32(lib, shape):
+    M, N, K = shape
+    a = torch.randn(M, K, device=DEV)
+    w = torch.randn(N, K, device=DEV)
+    out = torch.empty(M, N, device=DEV)
+    lib.gemm_f32(a, w, out)
+    close(out, plain.linear(a.cpu(), w.cpu()), torch.float32, scale=math.sqrt(K) * 4)
+    # a row's result does not depend on its neighbours
+    single = torch.empty(1, N, device=DEV)
+    lib.gemm_f32(a[M // 2:M // 2 + 1].contiguous(), w, single)
+    assert torch.equal(single[0], out[M // 2])
+
+
+# ---------------------------------------------------------------------------
+def rope_table(D, theta, positions):
+    angle = plain.rope_angles(list(range(positions)), D, theta)
+    return torch.cat([torch.cos(angle), torch.sin(angle)], dim=1).float().to(DEV)
+
+
+class PagedCache:
+    """A cache with a scrambled page table, filled with NaN so that a stray read or a
+    missed mask shows."""
+
+    def __init__(self, lengths, nkv, D, dtype, seed=0, extra_pages=3):
+        self.lengths = lengths
+        need = [(n + PAGE - 1) // PAGE for n in lengths]
+        self.n_pages = sum(need) + extra_pages
+        order = np.random.RandomState(seed).permutation(self.n_pages)
+        self.width = max(need) + 1
+        self.table = np.full((len(lengths), self.width), -1, dtype=np.int32)
+        at = 0
+        for b, n in enumerate(need):
+            self.table[b, :n] = order[at:at + n]
+            at += n
+        self.k = torch.full((self.n_pages, nkv, PAGE, D), float("nan"), device=DEV, dtype=dtype)
+        self.v = torch.full((self.n_pages, nkv, PAGE, D), float("nan"), device=DEV, dtype=dtype)
+        self.table_dev = torch.from_numpy(self.table).to(DEV)
+
+    def put(self, b, k, v):
+        """k, v: [len, nkv, D] for sequence b."""
+        for start in range(0, k.shape[0], PAGE):
+            page = self.table[b, start // PAGE]
+            n = min(PAGE, k.shape[0] - start)
+            self.k[page, :, :n] = k[start:start + n].transpose(0, 1).to(self.k.dtype)
+            self.v[page, :, :n] = v[start:start + n].transpose(0, 1).to(self.v.dtype)
+
+    def get(self, b, n):
+        pages = self.table[b, :(n + PAGE - 1) // PAGE]
+        k = torch.cat([self.k[p].transpose(0, 1) for p in pages])[:n]
+        v = torch.cat([self.v[p].transpose(0, 1) for p in pages])[:n]
+        return k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,D,use_norm,use_rope", [(6, 3, 48, True, True), (4, 4, 16, False, True),
+                                                        (8, 1, 256, True, False)])
+def test_qk_norm_rope_store(lib, dtype, nq, nkv, D, use_norm, use_rope):
+    theta, eps = 1e6, 1e-5
+    lengths_before = [70, 0, 130]
+    counts = [3, 5, 1]
+    N = sum(counts)
+    cache = PagedCache([a + c for a, c in zip(lengths_before, counts)], nkv, D, dtype, seed=1)
+    sentinel_k, sentinel_v = cache.k.clone(), cache.v.clone()
+    width = (nq + 2 * nkv) * D
+    qkv = torch.randn(2, N, width, device=DEV)
+    row_pos, row_seq = [], []
+    for b, (start, count) in enumerate(zip(lengths_before, counts)):
+        row_pos += list(range(start, start + count))
+        row_seq += [b] * count
+    row_pos[5], row_seq[5] = 0, -1         # a padding row in the middle is skipped
+    pos = torch.tensor(row_pos, dtype=torch.int32, device=DEV)
+    seq = torch.tensor(row_seq, dtype=torch.int32, device=DEV)
+    qn = (1 + 0.1 * torch.randn(D, device=DEV)) if use_norm else None
+    kn = (1 + 0.1 * torch.randn(D, device=DEV)) if use_norm else None
+    table = rope_table(D, theta, 256) if use_rope else None
+    q_out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=dtype)
+    lib.qk_norm_rope_store(qkv, qn, kn, eps, table, pos, seq, cache.table_dev, q_out, cache.k,
+                           cache.v, nq, nkv, D)
+    total = qkv.double().cpu().sum(0)
+    q = total[:, :nq * D].reshape(N, nq, D)
+    k = total[:, nq * D:(nq + nkv) * D].reshape(N, nkv, D)
+    v = total[:, (nq + nkv) * D:].reshape(N, nkv, D)
+    if use_norm:
+        q = plain.rms_norm(q, qn.cpu(), eps)
+        k = plain.rms_norm(k, kn.cpu(), eps)
+    if use_rope:
+        q = plain.rope(q, row_pos, theta)
+        k = plain.rope(k, row_pos, theta)
+    touched_k = torch.zeros_like(cache.k, dtype=torch.bool)
+    for r in range(N):
+        if row_seq[r] < 0:
+            assert torch.isnan(q_out[r].float()).all()
+            continue
+        close(q_out[r].reshape(nq, D), q[r], dtype, scale=q.abs().max().item())
+        page = cache.table[row_seq[r], row_pos[r] // PAGE]
+        close(cache.k[page, :, row_pos[r] % PAGE], k[r], dtype, scale=k.abs().max().item())
+        close(cache.v[page, :, row_pos[r] % PAGE], v[r], dtype, scale=v.abs().max().item())
+        touched_k[page, :, row_pos[r] % PAGE] = True
+    # nothing else in the cache changed (NaN sentinels compare by bits)
+    same_k = cache.k.view(torch.int16 if dtype == torch.bfloat16 else torch.int32) == \
+        sentinel_k.view(torch.int16 if dtype == torch.bfloat16 else torch.int32)
+    same_v = cache.v.view(torch.int16 if dtype == torch.bfloat16 else torch.int32) == \
+        sentinel_v.view(torch.int16 if dtype == torch.bfloat16 else torch.int32)
+    assert same_k[~touched_k].all() and same_v[~touched_k].all()
+    assert not same_k[touched_k].any()
+    # a layer that only reads another layer's cache writes nothing
+    again_k = cache.k.clone()
+    lib.qk_norm_rope_store(qkv, qn, kn, eps, table, pos, seq, cache.table_dev, q_out, cache.k,
+                           cache.v, nq, nkv, D, write_cache=False)
+    assert torch.equal(again_k.view(torch.uint8), cache.k.view(torch.uint8))
+
+
+def small_angle_vector_through_the_kernel(lib, dtype):
+    D = 128
+    table = rope_table(D, 1e6, 21)
+    basis = torch.zeros(21, 3 * D, device=DEV)
+    basis[:, :D // 2] = 1.0
+    cache = PagedCache([21], 1, D, dtype)
+    pos = torch.arange(21, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(21, dtype=torch.int32, device=DEV)
+    q_out = torch.empty(21, D, device=DEV, dtype=dtype)
+    lib.qk_norm_rope_store(basis, None, None, 1e-6, table, pos, seq, cache.table_dev, q_out,
+                           cache.k, cache.v, 1, 1, D)
+    return q_out.double().cpu()
+
+
+def test_rope_small_angle_reference_vector_on_the_gpu(lib):
+    """operators/tests/operators_cuda_bf16_contract_test.cu:372-415."""
+    out = small_angle_vector_through_the_kernel(lib, torch.float32)
+    for p in range(21):
+        for i in range(64):
+            angle = p / (1e6 ** (2.0 * i / 128))
+            assert abs(out[p, i].item() - math.cos(angle)) < 2e-6
+            assert abs(out[p, i + 64].item() - math.sin(angle)) < 2e-6
+
+
+# ---------------------------------------------------------------------------
+def items_for(lib, starts, counts, group):
+    per = lib.attention_positions_per_item(group)
+    seq, row0, npos, row = [], [], [], 0
+    for b, count in enumerate(counts):
+        for p0 in range(0, count, per):
+            seq.append(b)
+            row0.append(row + p0)
+            npos.append(min(per, count - p0))
+        row += count
+    as_dev = lambda x: torch.tensor(x, dtype=torch.int32, device=DEV)
+    return as_dev(seq), as_dev(row0), as_dev(npos), len(seq)
+
+
+def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
+                  boost=None):
+    """Fill a paged cache with random keys and values, run the kernel for the last
+    `counts[b]` positions of each sequence, return (kernel output, plain output)."""
+    torch.manual_seed(seed)
+    lengths = [s + c for s, c in zip(starts, counts)]
+    cache = PagedCache(lengths, nkv, D, dtype, seed=seed)
+    N = sum(counts)
+    q = torch.randn(N, nq, D, device=DEV).to(dtype)
+    ks, vs = [], []
+    for b, n in enumerate(lengths):
+        k = torch.randn(n, nkv, D, device=DEV).to(dtype)
+        v = torch.randn(n, nkv, D, device=DEV).to(dtype)
+        if boost is not None and boost[0] == b:
+            _, key_index, row_index, factor = boost
+            k[key_index] = (q[row_index, :nkv].float() * factor / D).to(dtype)
+        cache.put(b, k, v)
+        ks.append(k)
+        vs.append(v)
+    row_pos, row_seq = [], []
+    for b, (s, c) in enumerate(zip(starts, counts)):
+        row_pos += list(range(s, s + c))
+        row_seq += [b] * c
+    pos = torch.tensor(row_pos, dtype=torch.int32, device=DEV)
+    seq = torch.tensor(row_seq, dtype=torch.int32, device=DEV)
+    group = nq // nkv
+    item_seq, item_row0, item_npos, n_items = items_for(lib, starts, counts, group)
+    out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=dtype)
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.full((N * nq * splits * D,), float("nan"), device=DEV)
+        part_ml = torch.full((N * nq * splits * 2,), float("nan"), device=DEV)
+    lib.attention(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0, item_npos,
+                  n_items, pos, seq, cache.table_dev, out, nq, nkv, D, window=window,
+                  n_splits=splits, part_o=part_o, part_ml=part_ml)
+    expected = torch.empty(N, nq, D, dtype=torch.float64)
+    row = 0
+    for b, (s, c) in enumerate(zip(starts, counts)):
+        n = s + c
+        full_q = torch.zeros(n, nq, D, dtype=torch.float64)
+        full_q[s:] = q[row:row + c].double().cpu()
+        ref = plain.attention(full_q, ks[b].double().cpu(), vs[b].double().cpu(), window=window)
+        expected[row:row + c] = ref[s:]
+        row += c
+    return out.reshape(N, nq, D), expected
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,D", [(4, 2, 16), (6, 3, 48), (8, 1, 32), (4, 4, 128),
+                                      (20, 1, 64), (3, 1, 256), (32, 8, 128)])
+def test_attention_prefill_unequal_sequences(lib, dtype, nq, nkv, D):
+    """Whole prompts of unequal lengths (1, a page boundary, beyond one page) and a
+    chunk appended to 70 cached tokens, in one launch."""
+    out, expected = run_attention(lib, dtype, nq, nkv, D, starts=[0, 0, 0, 70, 0],
+                                  counts=[1, 64, 131, 9, 17])
+    close(out, expected, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,D,splits", [(4, 2, 16, 1), (8, 1, 32, 3), (32, 8, 128, 4),
+                                             (6, 3, 48, 8), (20, 1, 64, 2)])
+def test_attention_decode_with_splits(lib, dtype, nq, nkv, D, splits):
+    """One position per sequence; lengths around the split and page boundaries (the
+    reference sweeps 1, 2, 8, 9, 16, 17, ... across its own branch thresholds,
+    operators/tests/operators_cuda_attention_precision_test.cu:183)."""
+    starts = [0, 1, 62, 63, 64, 127, 128, 300, 8]
+    out, expected = run_attention(lib, dtype, nq, nkv, D, starts=starts, counts=[1] * len(starts),
+                                  splits=splits)
+    close(out, expected, dtype)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_finds_a_far_key_among_hundreds(lib, dtype):
+    """One early key is made to match the last query (score ~ 25 above the rest): the
+    output must be that key's value, in prefill and in split decode."""
+    nq, nkv, D = 4, 2, 64
+    for starts, counts, splits, row in (([0], [400], 1, 399), ([399], [1], 5, 0)):
+        out, expected = run_attention(lib, dtype, nq, nkv, D, starts, counts, splits=splits,
+                                      boost=(0, 3, row, 200.0), seed=4)
+        close(out, expected, dtype)
+        # the boosted key dominates head 0's softmax
+        assert (out[row, 0].double().cpu() - expected[row, 0]).abs().max() < 0.05
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 7, 64, 100])
+def test_attention_window_edge(lib, dtype, window):
+    """A standout key exactly at the window's edge counts; one step further it does not."""
+    nq, nkv, D = 2, 1, 32
+    n = 230
+    for key_index in (n - window, n - window - 1):          # inside, just outside
+        if key_index < 0:
+            continue
+        for starts, counts, splits, row in (([0], [n], 1, n - 1), ([n - 1], [1], 3, 0)):
+            out, expected = run_attention(lib, dtype, nq, nkv, D, starts, counts, window=window,
+                                          splits=splits, boost=(0, key_index, row, 300.0), seed=9)
+            close(out, expected, dtype)
+
+
+def test_attention_refuses_sizes_it_cannot_run(lib):
+    from edge_infer_amd.csrc.lib import KernelError
+    with pytest.raises(KernelError, match="multiple of 16"):
+        run_attention(lib, torch.float32, 2, 1, 24, [0], [4])
+    with pytest.raises(KernelError, match="multiple of 16"):
+        run_attention(lib, torch.float32, 2, 1, 512, [0], [4])
+
+
+# ---------------------------------------------------------------------------
+def test_argmax_ties_and_nan(lib):
+    rows = torch.tensor([[2, 1, 0, -1], [-3, 5, 1, 0], [0, -1, 4, 2], [1, 3, 3, 2],
+                         [float("nan"), -5, -5, -7]], dtype=torch.float32, device=DEV)
+    tokens = torch.empty(5, dtype=torch.int32, device=DEV)
+    prob = torch.empty(5, device=DEV)
+    lib.argmax(rows, tokens, prob)
+    assert tokens.tolist() == [0, 1, 2, 1, 1]
+    assert prob.tolist() == [1.0] * 5
+    big = torch.randn(3, 151936, device=DEV)
+    big[1, 150000] = 9.0
+    big[1, 77] = 9.0
+    tokens = torch.empty(3, dtype=torch.int32, device=DEV)
+    lib.argmax(big, tokens)
+    assert tokens.tolist() == [int(big[0].argmax()), 77, int(big[2].argmax())]
+
+
+def test_sample_reference_distribution(lib):
+    """operators/tests/operators_cuda_sampling_test.cu:133-198: logits log{.4,.3,.2,.1}, 2048
+    seeded draws for three (T, p, k): support, reported probability within 2e-5 of the
+    filtered softmax, frequencies within 0.05; and every draw equals the plain sampler's."""
+    logits = np.log(np.array([0.4, 0.3, 0.2, 0.1], dtype=np.float32))
+    rows = 2048
+    dev = torch.from_numpy(np.tile(logits, (rows, 1))).to(DEV)
+    streams = torch.zeros(rows, dtype=torch.int32, device=DEV)
+    counters = torch.arange(rows, dtype=torch.int32, device=DEV)
+    for temperature, top_p, top_k in [(1.0, 1.0, 2), (1.0, 0.65, 4), (0.75, 0.95, 3)]:
+        tokens = torch.empty(rows, dtype=torch.int32, device=DEV)
+        prob = torch.empty(rows, device=DEV)
+        lib.sample(dev, temperature, top_p, top_k, 1234567, streams, counters, tokens, prob)
+        order, expected = plain.filtered_distribution(logits, temperature, top_p, top_k)
+        table = dict(zip(order.tolist(), expected.tolist()))
+        got, got_p = tokens.tolist(), prob.tolist()
+        counts = {t: 0 for t in table}
+        for draw, (token, p) in enumerate(zip(got, got_p)):
+            assert token in table and abs(p - table[token]) < 2e-5
+            counts[token] += 1
+            assert token == plain.sample(logits, temperature, top_p, top_k,
+                                         plain.uniform(1234567, 0, draw))
+        assert max(abs(counts[t] / rows - table[t]) for t in table) < 0.05
+
+
+def test_sample_large_vocabulary_matches_plain(lib):
+    V = 151936
+    g = torch.Generator().manual_seed(3)
+    logits = (torch.randn(6, V, generator=g) * 2.5)
+    logits[2, :5000] = 6.0                         # thousands of ties around the threshold
+    logits[3, 100:104] = 30.0                      # ties at the very top
+    logits[4, :] = -1.0                            # everything equal
+    logits[5, 17] = float("nan")
+    dev = logits.to(DEV)
+    streams = torch.tensor([0, 1, 2, 3, 4, 5], dtype=torch.int32, device=DEV)
+    counters = torch.tensor([0, 5, 9, 1, 2, 3], dtype=torch.int32, device=DEV)
+    for temperature, top_p, top_k in [(0.8, 0.95, 50), (1.3, 1.0, 1024), (0.7, 0.5, 20),
+                                      (1.0, 1.0, 3)]:
+        tokens = torch.empty(6, dtype=torch.int32, device=DEV)
+        lib.sample(dev, temperature, top_p, top_k, 42, streams, counters, tokens)
+        for r in range(6):
+            u = plain.uniform(42, int(streams[r]), int(counters[r]))
+            assert tokens[r].item() == plain.sample(logits[r].numpy(), temperature, top_p, top_k, u), \
+                (r, temperature, top_p, top_k)
+
+
+def test_sample_refuses_bad_policies(lib):
+    from edge_infer_amd.csrc.lib import KernelError
+    logits = torch.zeros(1, 5000, device=DEV)
+    ints = torch.zeros(1, dtype=torch.int32, device=DEV)
+    for temperature, top_p, top_k in [(1.0, 0.0, 5), (1.0, 1.5, 5), (1.0, 0.9, 0), (1.0, 0.9, 1025),
+                                      (0.0, 0.9, 5)]:
+        with pytest.raises(KernelError):
+            lib.sample(logits, temperature, top_p, top_k, 0, ints, ints, ints.clone())
