@@ -1,0 +1,177 @@
+"""Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+Prints one JSON line.  `value` is decoded tokens per second at the given batch after
+512-token prompts (one step = one decode step of the whole batch: the model, greedy
+sampling, and the tokens fed back).  `prefill` is one prompt of 2,048 tokens;
+`roofline` prices the decode step against HBM bandwidth (every weight it uses once,
+plus the cache of the live requests); `points` hold decode at batch 1 and 64.
+Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
+ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+"""
+import argparse
+import json
+import sys
+import time
+from pathlib import Path
+
+sys.path.insert(0, str(Path(__file__).resolve().parent))
+
+HBM_PEAK_GBS = 8000.0
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}
+PROMPT = 512
+PREFILL_TOKENS = 2048
+CONTEXT = 4096
+
+
+def model_config(layers):
+    import edge_infer_amd as ei
+    return ei.Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=layers,
+                          num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                          intermediate_size=12288, max_position_embeddings=40960,
+                          bos_token_id=151643, eos_token_id=151645, rms_norm_eps=1e-6,
+                          rope_theta=1e6, tie_word_embeddings=False)
+
+
+def step_bytes(cfg, batch, context, itemsize):
+    """Bytes a decode step has to read: layer and head weights once, the live cache."""
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    layer = (Q + 2 * KV) * H + H * Q + 3 * I * H
+    weights = itemsize * (cfg.num_hidden_layers * layer + V * H)
+    cache = itemsize * 2 * cfg.num_hidden_layers * KV * batch * context
+    return weights + cache
+
+
+def prefill_flops(cfg, tokens):
+    H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    layer = 2 * tokens * ((Q + 2 * KV) * H + H * Q + 3 * I * H)
+    attention = 2 * 2 * cfg.num_attention_heads * cfg.head_dim * tokens * (tokens + 1) / 2
+    return cfg.num_hidden_layers * (layer + attention) + 2 * V * H
+
+
+def synthetic_prompts(cfg, batch, length, seed):
+    import torch
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, cfg.vocab_size, (batch, length), generator=g).tolist()
+
+
+def measure_decode(model, cfg, batch, steps, warmup):
+    """(ms per step, mean context during the timed steps)."""
+    import torch
+    import edge_infer_amd as ei
+    from edge_infer_amd.sampling import Sampler, SamplingParams
+    session = ei.Session(model, max_tokens=batch * CONTEXT, max_seqs=batch,
+                         max_seq_tokens=CONTEXT)
+    sampler = Sampler(model.device)
+    greedy = SamplingParams(temperature=0.0)
+    prompts = synthetic_prompts(cfg, batch, PROMPT, seed=100 + batch)
+    slots = [session.begin() for _ in range(batch)]
+    logits = session.step([(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)], copy=False)
+    tokens = sampler(logits, greedy, [], [])
+
+    def run(count):
+        nonlocal tokens
+        for _ in range(count):
+            logits = session.step([(s, [t], [0]) for s, t in zip(slots, tokens)], copy=False)
+            tokens = sampler(logits, greedy, [], [])
+
+    run(warmup)
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    run(steps)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    context = PROMPT + warmup + (steps + 1) / 2
+    for s in slots:
+        session.end(s)
+    del session
+    torch.cuda.empty_cache()
+    return 1000.0 * elapsed / steps, context
+
+
+def measure_prefill(model, cfg, repeats=3):
+    import torch
+    import edge_infer_amd as ei
+    session = ei.Session(model, max_tokens=PREFILL_TOKENS, max_seqs=1)
+    prompt = synthetic_prompts(cfg, 1, PREFILL_TOKENS, seed=7)[0]
+    best = None
+    for _ in range(repeats + 1):
+        slot = session.begin()
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        session.step([(slot, prompt, [PREFILL_TOKENS - 1])], copy=False)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        session.end(slot)
+        best = elapsed if best is None else min(best, elapsed)
+    del session
+    torch.cuda.empty_cache()
+    return 1000.0 * best
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=36,
+                        help="layers of the model (36 is the full Qwen3-8B shape)")
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--skip-points", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+    import edge_infer_amd as ei
+    cfg = model_config(args.layers)
+    model = ei.random_model(cfg, seed=2, dtype=args.dtype)
+    torch.cuda.synchronize()
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+
+    ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
+    value = args.batch * 1000.0 / ms_step
+    achieved = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9
+    prefill_ms = measure_prefill(model, cfg)
+    flops = prefill_flops(cfg, PREFILL_TOKENS)
+    points = {}
+    if not args.skip_points:
+        for name, batch in (("decode_b1", 1), ("decode_b64", 64)):
+            ms, _ = measure_decode(model, cfg, batch, max(8, args.steps // 2), args.warmup)
+            points[name] = round(batch * 1000.0 / ms, 1)
+    from edge_infer_amd.csrc import lib
+    record = {
+        "metric": "decode tokens/s, Qwen3-8B shape, batch 8 after 512-token prompts",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic token ids, seeded random weights N(0, 0.02)",
+        "config": {
+            "model": "Qwen3-8B shape", "layers": args.layers, "layers_full_model": 36,
+            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
+            "tie_word_embeddings": False, "global_batch": args.batch, "prompt_len": PROMPT,
+            "context_capacity": CONTEXT, "seq_len": round(context), "parallelism": "single GPU",
+            "kernels": "+".join(lib.loaded_libraries()),
+        },
+        "prefill": {"value": round(PREFILL_TOKENS * 1000.0 / prefill_ms, 1),
+                    "tokens": PREFILL_TOKENS, "ms": round(prefill_ms, 3),
+                    "frac": round(flops / (prefill_ms * 1e-3) / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": points,
+    }
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
