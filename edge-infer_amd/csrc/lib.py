@@ -9,6 +9,7 @@ these functions: if a library cannot be built or loaded the call raises.
 from __future__ import annotations
 
 import ctypes
+import os
 from ctypes import c_float, c_int, c_longlong, c_ulonglong, c_void_p
 from typing import Dict, Optional
 
@@ -41,9 +42,20 @@ _SIGNATURES = {
                          c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                          c_int, c_int, c_int, c_int, c_float, c_int, c_void_p],
     },
+    "attention_mfma": {
+        "ei_attn_decode_mfma_supported": [c_int, c_int],
+        "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                     c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                     c_int, c_int, c_float, c_int, c_void_p],
+    },
     "gemm_f32": {
         "ei_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_longlong, c_longlong,
                         c_longlong, c_void_p],
+    },
+    "gemm_bf16": {
+        "ei_skinny_gemm_splits": [c_int, c_int, c_int, c_int],
+        "ei_gemm_bf16_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                c_void_p],
     },
     "sampling": {
         "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
@@ -245,6 +257,40 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
     _check(lib, status, "attention")
 
 
+def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
+    return bool(library("attention_mfma").ei_attn_decode_mfma_supported(head_dim, group))
+
+
+def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,
+                          n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
+                          part_ml=None) -> None:
+    """bfloat16 decode attention on the matrix cores: one query row per sequence."""
+    lib = library("attention_mfma")
+    n = q.shape[0]
+    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
+        raise KernelError("attention_decode: q and out must be [rows, heads * head_dim]")
+    expect = (n_kv_heads, PAGE_TOKENS, head_dim)
+    if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
+        raise KernelError(f"attention_decode: pages must be [*, {expect}]")
+    if row_pos.numel() < n or row_seq.numel() < n or page_table.shape[0] < n:
+        raise KernelError("attention_decode: row metadata shorter than the rows")
+    if n_splits > 1:
+        if part_o is None or part_ml is None or part_o.numel() < n * n_heads * n_splits * head_dim \
+                or part_ml.numel() < n * n_heads * n_splits * 2:
+            raise KernelError("attention_decode: split scratch missing or too small")
+    if scale is None:
+        scale = head_dim ** -0.5
+    status = lib.ei_attention_decode_mfma(
+        _gpu(q, "q", torch.bfloat16), _gpu(k_pages, "k_pages", torch.bfloat16),
+        _gpu(v_pages, "v_pages", torch.bfloat16), _gpu(row_pos, "row_pos", torch.int32),
+        _gpu(row_seq, "row_seq", torch.int32), _gpu(page_table, "page_table", torch.int32),
+        page_table.shape[-1], _gpu(out, "out", torch.bfloat16),
+        None if part_o is None else _gpu(part_o, "part_o", torch.float32),
+        None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
+        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, _stream())
+    _check(lib, status, "attention_decode")
+
+
 def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     """out[M, N] = a[M, K] . w[N, K]^T in float32."""
     lib = library("gemm_f32")
@@ -289,3 +335,30 @@ def sample(logits, temperature, top_p, top_k, seed, streams, counters, tokens,
 # ---------------------------------------------------------------------------
 def has_skinny_gemm() -> bool:
     return "gemm_bf16" in build.available_libraries()
+
+
+_SKINNY_TARGET = int(os.environ.get("EDGE_INFER_SKINNY_BLOCKS", "0"))
+
+
+def skinny_gemm_splits(rows: int, n: int, k: int) -> int:
+    """K slices the weight-streaming product uses for [rows, k] x [n, k]^T."""
+    return library("gemm_bf16").ei_skinny_gemm_splits(rows, n, k, _SKINNY_TARGET)
+
+
+def skinny_gemm_ok(rows: int, k: int) -> bool:
+    return rows <= 64 and k % 8 == 0
+
+
+def gemm_bf16_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out[s, m, n] = sum over the s-th slice of K of x[m, :] . w[n, :] (float32), for at
+    most 64 rows; out.shape[0] says into how many slices K is cut."""
+    lib = library("gemm_bf16")
+    m, k = x.shape
+    n = w.shape[0]
+    if out.dim() != 3 or w.shape[1] != k or tuple(out.shape[1:]) != (m, n):
+        raise KernelError(f"gemm_bf16_skinny: shapes {list(x.shape)} x {list(w.shape)}^T -> "
+                          f"{list(out.shape)} do not agree")
+    status = lib.ei_gemm_bf16_skinny(_gpu(x, "x", torch.bfloat16), _gpu(w, "w", torch.bfloat16),
+                                     _gpu(out, "out", torch.float32), m, n, k, out.shape[0],
+                                     _stream())
+    _check(lib, status, "gemm_bf16_skinny")

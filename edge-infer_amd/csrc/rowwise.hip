@@ -60,6 +60,96 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
     dst[i] = ei::from_f32<TO>((row_values[i] * inv) * weight[i]);
 }
 
+// The same for widths that are a multiple of 4: 16-byte accesses, the row kept in
+// registers, up to 1024 threads a row so that few rows still have many loads in flight.
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 x = *reinterpret_cast<const float4*>(p);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Vec4<bf16_t> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
+    const uint2 x = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(x.x << 16); v[1] = __uint_as_float(x.x & 0xffff0000u);
+    v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
+    uint2 x;
+    x.x = static_cast<uint32_t>(ei::f32_to_bf16(v[0])) | (static_cast<uint32_t>(ei::f32_to_bf16(v[1])) << 16);
+    x.y = static_cast<uint32_t>(ei::f32_to_bf16(v[2])) | (static_cast<uint32_t>(ei::f32_to_bf16(v[3])) << 16);
+    *reinterpret_cast<uint2*>(p) = x;
+  }
+};
+
+template <typename TD, typename TO, bool HAS_DELTA, int CHUNKS>
+__global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
+                                       int nsplit, size_t split_stride,
+                                       const int32_t* __restrict__ rows,
+                                       const float* __restrict__ weight, float eps,
+                                       TO* __restrict__ out, int H, int write_residual) {
+  __shared__ float scratch[16];
+  const int row = blockIdx.x;
+  const int src = rows ? rows[row] : row;
+  const int quads = H / 4;
+  TO* dst = out + static_cast<size_t>(row) * H;
+  if (src < 0) {
+    const float zero[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int qd = threadIdx.x; qd < quads; qd += blockDim.x) Vec4<TO>::store(dst + qd * 4, zero);
+    return;
+  }
+  float* res = residual + static_cast<size_t>(src) * H;
+  float x[CHUNKS][4];
+  float sum = 0.f;
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    x[k][0] = x[k][1] = x[k][2] = x[k][3] = 0.f;
+    if (qd < quads) {
+      Vec4<float>::load(res + qd * 4, x[k]);
+      if (HAS_DELTA) {
+        const TD* d = delta + static_cast<size_t>(src) * H + qd * 4;
+        int s = 0;
+        for (; s + 4 <= nsplit; s += 4) {       // four independent loads in flight
+          float a[4], b[4], c[4], e[4];
+          Vec4<TD>::load(d + (s + 0) * split_stride, a);
+          Vec4<TD>::load(d + (s + 1) * split_stride, b);
+          Vec4<TD>::load(d + (s + 2) * split_stride, c);
+          Vec4<TD>::load(d + (s + 3) * split_stride, e);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[k][i] = (((x[k][i] + a[i]) + b[i]) + c[i]) + e[i];
+        }
+        for (; s < nsplit; ++s) {
+          float a[4];
+          Vec4<TD>::load(d + s * split_stride, a);
+#pragma unroll
+          for (int i = 0; i < 4; ++i) x[k][i] += a[i];
+        }
+        if (write_residual) Vec4<float>::store(res + qd * 4, x[k]);
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
+    }
+  }
+  const float total = ei::block_sum(sum, scratch);
+  const float inv = rsqrtf(total / static_cast<float>(H) + eps);
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) {
+      float w[4], y[4];
+      Vec4<float>::load(weight + qd * 4, w);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) y[i] = (x[k][i] * inv) * w[i];
+      Vec4<TO>::store(dst + qd * 4, y);
+    }
+  }
+}
+
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
                               TO* __restrict__ out, int I, size_t total) {
@@ -100,6 +190,27 @@ template <typename TD, typename TO>
 static void launch_add_rmsnorm(float* residual, const void* delta, int nsplit, size_t split_stride,
                                const int32_t* rows, const float* weight, float eps, void* out,
                                int N, int H, int write_residual, hipStream_t stream) {
+  if (H % 4 == 0 && (!delta || split_stride % 4 == 0)) {
+    const int quads = H / 4;
+    int threads = (quads + EI_WAVE - 1) / EI_WAVE * EI_WAVE;
+    if (threads > 1024) threads = 1024;
+    const int chunks = (quads + threads - 1) / threads;      // 1..4 for H <= 16384
+#define EI_NORM_VEC(C)                                                                         \
+  do {                                                                                         \
+    if (delta)                                                                                 \
+      add_rmsnorm_vec_kernel<TD, TO, true, C><<<N, threads, 0, stream>>>(                      \
+          residual, static_cast<const TD*>(delta), nsplit, split_stride, rows, weight, eps,    \
+          static_cast<TO*>(out), H, write_residual);                                           \
+    else                                                                                       \
+      add_rmsnorm_vec_kernel<TD, TO, false, C><<<N, threads, 0, stream>>>(                     \
+          residual, nullptr, 0, 0, rows, weight, eps, static_cast<TO*>(out), H, 0);            \
+  } while (0)
+    if (chunks == 1) EI_NORM_VEC(1);
+    else if (chunks == 2) EI_NORM_VEC(2);
+    else EI_NORM_VEC(4);
+#undef EI_NORM_VEC
+    return;
+  }
   const int threads = H >= 2048 ? 256 : (H >= 256 ? 128 : 64);
   const size_t lds = static_cast<size_t>(H) * sizeof(float);
   if (delta)

@@ -109,6 +109,27 @@ class DecoderModel:
                 limit = min(limit, table.max_positions)
         return limit
 
+    def capture_safe(self) -> bool:
+        """Whether a decode step may be captured in a HIP graph: every linear layer must
+        take the hand-written kernel for few rows (library products may record memset
+        nodes, which are not replayed reliably), and every mixer must say it is safe."""
+        def linears(obj, depth=0):
+            if isinstance(obj, Linear):
+                yield obj
+            elif depth < 3 and hasattr(obj, "__dict__"):
+                for value in vars(obj).values():
+                    yield from linears(value, depth + 1)
+        for layer in self.layers:
+            mixer = getattr(layer, "mixer", None)
+            if mixer is not None and not getattr(mixer, "capture_safe", False):
+                return False
+            for linear in linears(layer):
+                if linear.dtype == torch.bfloat16 and linear.in_features % 8:
+                    return False
+        if self.head.dtype == torch.bfloat16 and self.head.in_features % 8:
+            return False
+        return True
+
     def weight_bytes(self) -> int:
         seen, total = set(), 0
 

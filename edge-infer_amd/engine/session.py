@@ -20,22 +20,37 @@ from .batch import DeviceMeta, SeqStep, StepPlan
 
 
 class _Context(StepContext):
-    def __init__(self, session, **kwargs):
+    def __init__(self, session, fixed_context=None, **kwargs):
         super().__init__(**kwargs)
         self._session = session
+        self._fixed_context = fixed_context
 
     def decode_splits(self, n_kv_heads: int) -> int:
         """How many blocks share the key range of one (sequence, kv head) in decode:
         enough to put about two blocks on each of the 256 compute units, never more
-        than there are pages."""
-        pages = max(1, (self.max_context + PAGE_TOKENS - 1) // PAGE_TOKENS)
+        than there are pages.  A captured step fixes the count by the capacity (blocks
+        whose share of a short sequence is empty return at once)."""
+        context = self._fixed_context or self.max_context
+        pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
         wanted = (512 + self.n_seqs * n_kv_heads - 1) // (self.n_seqs * n_kv_heads)
         return max(1, min(wanted, pages, 32))
 
 
+class _CapturedDecode:
+    """A decode step of a fixed batch size, captured once as a HIP graph.  Everything
+    that changes from step to step (tokens, positions, page tables, which rows are
+    live) lives in its metadata buffer, which is filled before every replay."""
+
+    def __init__(self, device):
+        self.meta = DeviceMeta(device)
+        self.workspace = Workspace(device)
+        self.graph = None
+        self.logits = None
+
+
 class Session:
     def __init__(self, model, max_tokens: int, max_seqs: Optional[int] = None,
-                 max_seq_tokens: Optional[int] = None, seed: int = 0):
+                 max_seq_tokens: Optional[int] = None, seed: int = 0, graphs: bool = True):
         self.model = model
         self.device = model.device
         self.dtype = model.dtype
@@ -58,6 +73,11 @@ class Session:
         self.meta = DeviceMeta(self.device)
         self._item_sizes = model.attention_item_sizes()
         self.steps_run = 0
+        # decode steps are replayed from HIP graphs unless the model has an operation
+        # that is not safe to capture (see DecoderModel.capture_safe)
+        self.graphs = bool(graphs) and model.capture_safe()
+        self._captured: Dict[int, _CapturedDecode] = {}
+        self.graph_replays = 0
 
     # -- slots -----------------------------------------------------------
     def begin(self) -> int:
@@ -166,19 +186,57 @@ class Session:
         growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
         self.cache.check_growth(growth)          # raises before anything changes
         self.cache.grow(growth)
-        plan = StepPlan(seqs, item_sizes=self._item_sizes)
-        logits = self._run(plan, self.meta, self.workspace)
+        if self.graphs and all(seq.count == 1 for seq in seqs):
+            logits = self._run_captured(seqs)
+        else:
+            plan = StepPlan(seqs, item_sizes=self._item_sizes)
+            logits = self._run(plan, self.meta, self.workspace)
         self.cache.commit(growth)
         self.steps_run += 1
         return logits.clone() if copy else logits
 
-    def _run(self, plan: StepPlan, meta: DeviceMeta, workspace: Workspace) -> torch.Tensor:
+    def _context(self, plan, meta, workspace, fixed_context=None):
         slots = [seq.slot for seq in plan.seqs]
         tables = [self.cache.page_rows(group, slots, plan.n_seqs)
                   for group in range(len(self.cache.kv_pages))]
         meta.upload(plan, tables)
-        ctx = _Context(self, dtype=self.dtype, device=self.device, n_rows=plan.n_rows,
-                       n_seqs=plan.n_seqs, decode=plan.decode, meta=meta, cache=self.cache,
-                       workspace=workspace, max_context=plan.max_context)
+        ctx = _Context(self, fixed_context=fixed_context, dtype=self.dtype, device=self.device,
+                       n_rows=plan.n_rows, n_seqs=plan.n_seqs, decode=plan.decode, meta=meta,
+                       cache=self.cache, workspace=workspace, max_context=plan.max_context)
         ctx.sequences = plan.seqs
-        return self.model.forward(ctx)
+        return ctx
+
+    def _run(self, plan: StepPlan, meta: DeviceMeta, workspace: Workspace) -> torch.Tensor:
+        return self.model.forward(self._context(plan, meta, workspace))
+
+    def _run_captured(self, seqs: List[SeqStep]) -> torch.Tensor:
+        """A decode step through the graph of its batch-size bucket (powers of two).
+        The first step of a bucket runs eagerly on the bucket's own buffers and is then
+        captured; later steps only refresh the metadata and replay."""
+        live = len(seqs)
+        bucket = 1
+        while bucket < live:
+            bucket *= 2
+        plan = StepPlan(seqs, item_sizes=self._item_sizes, pad_seqs=bucket)
+        captured = self._captured.get(bucket)
+        if captured is None:
+            captured = self._captured[bucket] = _CapturedDecode(self.device)
+        ctx = self._context(plan, captured.meta, captured.workspace, fixed_context=self.capacity)
+        if captured.graph is None:
+            logits = self.model.forward(ctx)
+            torch.cuda.synchronize(self.device)
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                captured.logits = self.model.forward(ctx)
+            captured.graph = graph
+        else:
+            captured.graph.replay()
+            self.graph_replays += 1
+            logits = captured.logits
+        # the captured step computes the logits of every row; hand out the wanted ones
+        wanted = [index for index, seq in enumerate(seqs) if len(seq.want) > 0]
+        if len(wanted) == live:
+            return logits[:live]
+        if not wanted:
+            return logits[:0]
+        return logits[torch.tensor(wanted, device=self.device)]

@@ -19,6 +19,8 @@ from .registry import lookup
 
 
 class Attention:
+    capture_safe = True   # launches only this library's kernels; nothing allocates per step
+
     @classmethod
     def parameters(cls, spec, hidden):
         params = {
@@ -62,6 +64,10 @@ class Attention:
         self.position = positions(spec.position)   # shared table object
         self.group = spec.n_heads // spec.n_kv_heads
         self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
+        # the matrix-core kernels take bfloat16 with head sizes 64 and 128; every other
+        # case runs the generic kernel
+        self.fast_decode = (dtype == torch.bfloat16 and
+                            lib.attention_decode_mfma_supported(spec.head_dim, self.group))
 
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self):
@@ -88,11 +94,17 @@ class Attention:
                                     torch.float32)
                 part_ml = ctx.buffer("attn.part_ml", (n * spec.n_heads * splits * 2,),
                                      torch.float32)
-            item_seq, item_row0, item_npos, n_items = meta.decode_items()
-            lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
-                          meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
-                          spec.n_kv_heads, spec.head_dim, window=spec.window, scale=self.scale,
-                          n_splits=splits, part_o=part_o, part_ml=part_ml)
+            if self.fast_decode:
+                lib.attention_decode_mfma(q, k_pages, v_pages, meta.row_pos, meta.row_seq,
+                                          page_table, out, spec.n_heads, spec.n_kv_heads,
+                                          spec.head_dim, window=spec.window, scale=self.scale,
+                                          n_splits=splits, part_o=part_o, part_ml=part_ml)
+            else:
+                item_seq, item_row0, item_npos, n_items = meta.decode_items()
+                lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                              meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                              spec.n_kv_heads, spec.head_dim, window=spec.window,
+                              scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml)
         else:
             item_seq, item_row0, item_npos, n_items = meta.prefill_items(self.positions_per_item())
             lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,

@@ -2,8 +2,8 @@
 
 float32: the hand-written float32 kernel (no reduced-precision matrix mode).
 bfloat16: for up to `SKINNY_ROWS` rows the hand-written weight-streaming MFMA
-kernel, which returns float32 partial sums [splits, rows, out] that the consuming
-kernel adds up; for more rows the library matrix product (the reference multiplies
+kernel, which returns float32 partial sums [slices, rows, out] that the consuming
+kernel adds up while it reads them; for more rows the library matrix product (the reference multiplies
 through cuBLAS as well, operators/src/cuda/execution.cu:299-324).
 """
 from __future__ import annotations
@@ -24,14 +24,15 @@ class Linear:
         self.dtype = dtype
 
     def forward(self, ctx, x: torch.Tensor, out_name: str) -> torch.Tensor:
-        """x [N, in] of the step's storage type -> [N, out] (or float32 partial sums
-        [splits, N, out]); the result lives in the workspace buffer `out_name`."""
+        """x [N, in] of the step's storage type -> [N, out] in the storage type, or float32
+        partial sums [slices, N, out] when the few-rows kernel ran; the result lives in the
+        workspace buffer `out_name`."""
         rows = x.shape[0]
         if self.dtype == torch.float32:
             out = ctx.buffer(out_name, (rows, self.out_features), torch.float32)
             lib.gemm_f32(x, self.weight, out)
             return out
-        if rows <= SKINNY_ROWS and lib.has_skinny_gemm():
+        if lib.skinny_gemm_ok(rows, self.in_features):
             splits = lib.skinny_gemm_splits(rows, self.out_features, self.in_features)
             out = ctx.buffer(out_name + ".f32", (splits, rows, self.out_features), torch.float32)
             lib.gemm_bf16_skinny(x, self.weight, out)
@@ -47,11 +48,10 @@ class Linear:
         if self.dtype == torch.float32:
             lib.gemm_f32(x, self.weight, out)
             return out
-        if lib.has_skinny_gemm():
+        if self.in_features % 8 == 0 and rows <= 4 * SKINNY_ROWS:
             for start in range(0, rows, SKINNY_ROWS):
                 stop = min(rows, start + SKINNY_ROWS)
-                lib.gemm_bf16_skinny(x[start:stop], self.weight, out[start:stop].unsqueeze(0),
-                                     splits=1)
+                lib.gemm_bf16_skinny(x[start:stop], self.weight, out[start:stop].unsqueeze(0))
             return out
         low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)
         torch.matmul(x, self.weight.t(), out=low)

@@ -257,7 +257,7 @@ def items_for(lib, starts, counts, group):
 
 
 def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
-                  boost=None):
+                  boost=None, kernel="generic"):
     """Fill a paged cache with random keys and values, run the kernel for the last
     `counts[b]` positions of each sequence, return (kernel output, plain output)."""
     torch.manual_seed(seed)
@@ -288,9 +288,14 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     if splits > 1:
         part_o = torch.full((N * nq * splits * D,), float("nan"), device=DEV)
         part_ml = torch.full((N * nq * splits * 2,), float("nan"), device=DEV)
-    lib.attention(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0, item_npos,
-                  n_items, pos, seq, cache.table_dev, out, nq, nkv, D, window=window,
-                  n_splits=splits, part_o=part_o, part_ml=part_ml)
+    if kernel == "decode_mfma":
+        lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
+                                  cache.table_dev, out, nq, nkv, D, window=window,
+                                  n_splits=splits, part_o=part_o, part_ml=part_ml)
+    else:
+        lib.attention(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0, item_npos,
+                      n_items, pos, seq, cache.table_dev, out, nq, nkv, D, window=window,
+                      n_splits=splits, part_o=part_o, part_ml=part_ml)
     expected = torch.empty(N, nq, D, dtype=torch.float64)
     row = 0
     for b, (s, c) in enumerate(zip(starts, counts)):
@@ -353,6 +358,31 @@ def test_attention_window_edge(lib, dtype, window):
             out, expected = run_attention(lib, dtype, nq, nkv, D, starts, counts, window=window,
                                           splits=splits, boost=(0, key_index, row, 300.0), seed=9)
             close(out, expected, dtype)
+
+
+@pytest.mark.parametrize("nq,nkv,D,splits", [(32, 8, 128, 1), (32, 8, 128, 4), (8, 8, 64, 3),
+                                             (6, 2, 128, 2), (20, 1, 64, 5), (16, 1, 128, 32),
+                                             (2, 1, 64, 1)])
+def test_attention_decode_on_the_matrix_cores(lib, nq, nkv, D, splits):
+    """The bfloat16 decode kernel: lengths around tile (16), page (64) and slice
+    boundaries, group ratios that fill a head block partly, more slices than pages."""
+    starts = [0, 1, 14, 15, 16, 62, 63, 64, 127, 128, 300, 1029, 8]
+    out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, starts=starts,
+                                  counts=[1] * len(starts), splits=splits, kernel="decode_mfma")
+    close(out, expected, torch.bfloat16)
+
+
+@pytest.mark.parametrize("window", [1, 7, 64, 100])
+def test_attention_decode_on_the_matrix_cores_window_and_far_key(lib, window):
+    nq, nkv, D, n = 8, 2, 128, 230
+    for key_index in (n - window, n - window - 1):
+        out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [n - 1], [1], window=window,
+                                      splits=3, boost=(0, key_index, 0, 300.0), seed=9,
+                                      kernel="decode_mfma")
+        close(out, expected, torch.bfloat16)
+    out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [899], [1], splits=6,
+                                  boost=(0, 3, 0, 200.0), seed=4, kernel="decode_mfma")
+    close(out, expected, torch.bfloat16)
 
 
 def test_attention_refuses_sizes_it_cannot_run(lib):
@@ -434,3 +464,48 @@ def test_sample_refuses_bad_policies(lib):
                                       (0.0, 0.9, 5)]:
         with pytest.raises(KernelError):
             lib.sample(logits, temperature, top_p, top_k, 0, ints, ints, ints.clone())
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64])
+@pytest.mark.parametrize("N,K", [(381, 96), (200, 200), (96, 256), (4096, 1024), (1000, 1384)])
+def test_gemm_bf16_skinny(lib, M, N, K):
+    """The weight-streaming product for few rows: every slice count it may choose, widths
+    that are no multiple of the tile, and the same row alone or among others."""
+    torch.manual_seed(M * 7 + N)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    w = torch.randn(N, K, device=DEV).to(torch.bfloat16)
+    expected = plain.linear(x.cpu(), w.cpu())
+    chosen = lib.skinny_gemm_splits(M, N, K)
+    tile = 128 if M > 32 else 256
+    tiles = (K + tile - 1) // tile
+    candidates = {1, chosen}
+    for s in range(2, tiles + 1):            # every slice count that leaves no slice empty
+        per = (tiles + s - 1) // s
+        if (tiles + per - 1) // per == s:
+            candidates.add(s)
+    results = {}
+    for splits in sorted(candidates):
+        out = torch.full((splits, M, N), float("nan"), device=DEV)
+        lib.gemm_bf16_skinny(x, w, out)
+        err = (out.double().cpu().sum(0) - expected).abs().max().item()
+        assert err <= 2e-6 * math.sqrt(K) * 16, f"splits {splits}: max error {err:.3e}"
+        results[splits] = out
+    # a row gives the same bits alone as inside a batch of up to 16 rows (the same tile
+    # shape and slice count, hence the same order of accumulation)
+    if M <= 16 and lib.skinny_gemm_splits(1, N, K) == chosen:
+        single = torch.empty((chosen, 1, N), device=DEV)
+        lib.gemm_bf16_skinny(x[M // 2:M // 2 + 1].contiguous(), w, single)
+        assert torch.equal(single[:, 0], results[chosen][:, M // 2])
+
+
+def test_gemm_bf16_skinny_refuses_what_it_cannot_run(lib):
+    from edge_infer_amd.csrc.lib import KernelError
+    w = torch.zeros(32, 100, device=DEV, dtype=torch.bfloat16)
+    x = torch.zeros(2, 100, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="multiple of 8"):
+        lib.gemm_bf16_skinny(x, w, torch.empty(1, 2, 32, device=DEV))
+    w = torch.zeros(32, 96, device=DEV, dtype=torch.bfloat16)
+    x = torch.zeros(65, 96, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="1..64"):
+        lib.gemm_bf16_skinny(x, w, torch.empty(1, 65, 32, device=DEV))
