@@ -214,6 +214,190 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   }
 }
 
+// Prefill: a block of four waves owns 64 consecutive positions of one sequence and one query
+// head; each wave keeps 16 query rows as an MFMA operand in registers and walks the key
+// pages of the sequence.  A page of keys goes to LDS as stored, a page of values goes to LDS
+// transposed ([d][key]) so that both products read 8-element runs along their contraction
+// index.  Scores are computed transposed (S^T = K Q^T): lane (c, n) then holds, for query
+// row n, the keys 4c..4c+3 of every 16-key block, which is exactly an A-operand register
+// of P for the second product once two blocks are packed together, so the probabilities
+// never leave the registers.  Softmax state is float32; probabilities are rounded to
+// bfloat16 for the value product (the reference's prefill kernel does the same,
+// operators/src/cuda/kernels/flash_attn_prefill.cu:240).
+template <int D>
+__global__ void __launch_bounds__(kThreads)
+attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
+                    const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
+                    const int32_t* __restrict__ item_row0, const int32_t* __restrict__ item_npos,
+                    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ page_table,
+                    int table_width, bf16_t* __restrict__ out, int nq, int nkv, int window,
+                    float scale) {
+  constexpr int DJ = D / 32;             // MFMA steps over d for the scores
+  constexpr int DB = D / 16;             // 16-wide output blocks over d
+  constexpr int KS = D + 8;              // LDS stride of a key row (elements)
+  constexpr int VS = EI_PAGE + 8;        // LDS stride of a transposed value row
+  constexpr int CI = D / 32;             // 16-byte chunks per thread per page (D/8 * 64 / 256)
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[EI_PAGE * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * VS];
+
+  const int item = blockIdx.x, head = blockIdx.y;
+  const int seq = item_seq[item];
+  if (seq < 0) return;
+  const int row0 = item_row0[item], npos = item_npos[item];
+  const int G = nq / nkv, g = head / G;
+  const int t = threadIdx.x, wave = t / EI_WAVE, lane = t % EI_WAVE;
+  const int r16 = lane & 15, c = lane >> 4;
+
+  // this lane's query row (as column n of S^T) and its position
+  const int my_row = wave * 16 + r16;
+  const bool row_valid = my_row < npos;
+  const int pos_r = row_valid ? row_pos[row0 + my_row] : -1;
+  bf16x8 q_reg[DJ];
+#pragma unroll
+  for (int j = 0; j < DJ; ++j) {
+    uint4 z = uint4{0u, 0u, 0u, 0u};
+    if (row_valid)
+      z = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(row0 + my_row) * nq + head) * D +
+                                          j * 32 + c * 8);
+    q_reg[j] = *reinterpret_cast<bf16x8*>(&z);
+  }
+
+  const int first_pos = row_pos[row0], last_pos = row_pos[row0 + npos - 1];
+  const int lo_key = window > 0 ? max(0, first_pos - window + 1) : 0;
+  const int lo_page = lo_key / EI_PAGE, hi_page = last_pos / EI_PAGE;
+
+  float m_run = kLowest, l_run = 0.f;
+  f32x4 o_acc[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db) o_acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // global -> register staging of a page: thread t takes key t/4, chunks (t%4) + 4*i
+  const int ld_key = t >> 2, ld_dc = t & 3;
+  uint4 k_stage[CI], v_stage[CI];
+  auto load_page = [&](int page_index) {
+    const int phys = page_table[static_cast<size_t>(seq) * table_width + page_index];
+    if (phys < 0) {                       // released by the window: every key is masked
+#pragma unroll
+      for (int i = 0; i < CI; ++i) k_stage[i] = v_stage[i] = uint4{0u, 0u, 0u, 0u};
+      return;
+    }
+    const size_t base = ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D;
+    const bool live = page_index * EI_PAGE + ld_key <= last_pos;   // later slots: stale bytes
+#pragma unroll
+    for (int i = 0; i < CI; ++i) {
+      const int dc = ld_dc + 4 * i;
+      k_stage[i] = live ? *reinterpret_cast<const uint4*>(k_pages + base + dc * 8)
+                        : uint4{0u, 0u, 0u, 0u};
+      v_stage[i] = live ? *reinterpret_cast<const uint4*>(v_pages + base + dc * 8)
+                        : uint4{0u, 0u, 0u, 0u};
+    }
+  };
+  auto store_page = [&]() {
+#pragma unroll
+    for (int i = 0; i < CI; ++i) {
+      const int dc = ld_dc + 4 * i;
+      *reinterpret_cast<uint4*>(&k_lds[ld_key * KS + dc * 8]) = k_stage[i];
+      const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v_lds[(dc * 8 + 2 * e) * VS + ld_key] = static_cast<bf16_t>(w[e] & 0xffffu);
+        v_lds[(dc * 8 + 2 * e + 1) * VS + ld_key] = static_cast<bf16_t>(w[e] >> 16);
+      }
+    }
+  };
+
+  load_page(lo_page);
+  for (int page = lo_page; page <= hi_page; ++page) {
+    __syncthreads();                      // the previous page's reads are done
+    store_page();
+    __syncthreads();
+    if (page < hi_page) load_page(page + 1);
+    const int key_base = page * EI_PAGE;
+
+    // S^T blocks: lane (c, n) holds keys key_base + kb*16 + 4c + r for query row n
+    f32x4 s[4];
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+      s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < DJ; ++j) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+            &k_lds[(kb * 16 + r16) * KS + j * 32 + c * 8]);
+        s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_reg[j], s[kb], 0, 0, 0);
+      }
+    }
+    float tile_max = kLowest;
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int key = key_base + kb * 16 + 4 * c + r;
+        const bool visible = row_valid && key <= pos_r && (window <= 0 || key > pos_r - window);
+        const float v = visible ? s[kb][r] * scale : -INFINITY;
+        s[kb][r] = v;
+        tile_max = fmaxf(tile_max, v);
+      }
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, EI_WAVE));
+    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, EI_WAVE));
+    const float m_new = fmaxf(m_run, tile_max);
+    const float alpha = expf(m_run - m_new);
+    float tile_sum = 0.f;
+    bf16x8 p_reg[2];                      // A operand of P for the two 32-key steps
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16_t packed[8];
+#pragma unroll
+      for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float p = expf(s[2 * ks + half][r] - m_new);
+          tile_sum += p;
+          packed[half * 4 + r] = ei::f32_to_bf16(p);
+        }
+      p_reg[ks] = *reinterpret_cast<bf16x8*>(packed);
+    }
+    tile_sum += __shfl_xor(tile_sum, 16, EI_WAVE);
+    tile_sum += __shfl_xor(tile_sum, 32, EI_WAVE);
+    l_run = l_run * alpha + tile_sum;
+    m_run = m_new;
+    // the output rows of this lane are query rows 4c + r: fetch their factors
+    float a_row[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) a_row[r] = __shfl(alpha, 4 * c + r, EI_WAVE);
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o_acc[db][r] *= a_row[r];
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks) {
+        // values: lane (n = d column, c) supplies keys ks*32 + {4c..4c+3} and +16
+        const bf16_t* vrow = &v_lds[(db * 16 + r16) * VS + ks * 32 + 4 * c];
+        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        uint4 both = uint4{lo.x, lo.y, hi.x, hi.y};
+        o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            p_reg[ks], *reinterpret_cast<bf16x8*>(&both), o_acc[db], 0, 0, 0);
+      }
+    }
+  }
+
+  // lane (c, n) holds O[query row 4c + r][d = db*16 + n]
+  float inv_row[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float l = __shfl(l_run, 4 * c + r, EI_WAVE);
+    inv_row[r] = l > 0.f ? 1.f / l : 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int orow = wave * 16 + 4 * c + r;
+    if (orow >= npos) continue;
+    bf16_t* dst = out + (static_cast<size_t>(row0 + orow) * nq + head) * D;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) dst[db * 16 + r16] = ei::from_f32<bf16_t>(o_acc[db][r] * inv_row[r]);
+  }
+}
+
 // One wave per (row, head): o = sum_s o_s e^{m_s - m} / sum_s l_s e^{m_s - m}.
 __global__ void attn_merge_kernel(const float* __restrict__ part_o,
                                   const float* __restrict__ part_ml,
@@ -249,6 +433,39 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
 }
 
 }  // namespace
+
+// Positions of one sequence that a prefill work item of this file holds.
+extern "C" int ei_attn_prefill_mfma_positions() { return 64; }
+
+// q, out: [N, nq, D] bfloat16; items: (sequence, first packed row, up to 64 positions).
+extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, const void* v_pages,
+                                         const int32_t* item_seq, const int32_t* item_row0,
+                                         const int32_t* item_npos, int n_items,
+                                         const int32_t* row_pos, const int32_t* page_table,
+                                         int table_width, void* out, int nq, int nkv, int D,
+                                         int window, float scale, hipStream_t stream) {
+  EI_REQUIRE(n_items > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes");
+  EI_REQUIRE(D == 64 || D == 128, "attention_prefill: this kernel takes head_dim 64 or 128");
+  EI_REQUIRE(q && k_pages && v_pages && item_seq && item_row0 && item_npos && row_pos &&
+                 page_table && out && table_width > 0,
+             "attention_prefill: null pointer");
+  EI_REQUIRE(window >= 0, "attention_prefill: negative window");
+  EI_REQUIRE(nq <= 65535, "attention_prefill: too many heads");
+  dim3 grid(n_items, nq);
+  const bf16_t* qq = static_cast<const bf16_t*>(q);
+  const bf16_t* kk = static_cast<const bf16_t*>(k_pages);
+  const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
+  bf16_t* oo = static_cast<bf16_t*>(out);
+  if (D == 64)
+    attn_prefill_kernel<64><<<grid, kThreads, 0, stream>>>(qq, kk, vv, item_seq, item_row0,
+                                                           item_npos, row_pos, page_table,
+                                                           table_width, oo, nq, nkv, window, scale);
+  else
+    attn_prefill_kernel<128><<<grid, kThreads, 0, stream>>>(qq, kk, vv, item_seq, item_row0,
+                                                            item_npos, row_pos, page_table,
+                                                            table_width, oo, nq, nkv, window, scale);
+  EI_LAUNCH_CHECK();
+}
 
 // Whether the decode kernel of this file takes a head size and group ratio.
 extern "C" int ei_attn_decode_mfma_supported(int D, int G) {

@@ -44,6 +44,10 @@ _SIGNATURES = {
     },
     "attention_mfma": {
         "ei_attn_decode_mfma_supported": [c_int, c_int],
+        "ei_attn_prefill_mfma_positions": [],
+        "ei_attention_prefill_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
+                                      c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
+                                      c_int, c_int, c_float, c_void_p],
         "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_int, c_void_p],
@@ -259,6 +263,36 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
 
 def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
     return bool(library("attention_mfma").ei_attn_decode_mfma_supported(head_dim, group))
+
+
+def attention_prefill_mfma_positions() -> int:
+    return library("attention_mfma").ei_attn_prefill_mfma_positions()
+
+
+def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
+                           page_table, out, n_heads, n_kv_heads, head_dim, window=None,
+                           scale=None) -> None:
+    """bfloat16 prefill attention on the matrix cores; items hold up to 64 positions."""
+    lib = library("attention_mfma")
+    n = q.shape[0]
+    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
+        raise KernelError("attention_prefill: q and out must be [rows, heads * head_dim]")
+    expect = (n_kv_heads, PAGE_TOKENS, head_dim)
+    if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
+        raise KernelError(f"attention_prefill: pages must be [*, {expect}]")
+    if item_seq.numel() < n_items or item_row0.numel() < n_items or item_npos.numel() < n_items:
+        raise KernelError("attention_prefill: work item arrays shorter than n_items")
+    if scale is None:
+        scale = head_dim ** -0.5
+    status = lib.ei_attention_prefill_mfma(
+        _gpu(q, "q", torch.bfloat16), _gpu(k_pages, "k_pages", torch.bfloat16),
+        _gpu(v_pages, "v_pages", torch.bfloat16), _gpu(item_seq, "item_seq", torch.int32),
+        _gpu(item_row0, "item_row0", torch.int32), _gpu(item_npos, "item_npos", torch.int32),
+        n_items, _gpu(row_pos, "row_pos", torch.int32),
+        _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
+        _gpu(out, "out", torch.bfloat16), n_heads, n_kv_heads, head_dim, int(window or 0),
+        float(scale), _stream())
+    _check(lib, status, "attention_prefill")
 
 
 def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,

@@ -66,11 +66,13 @@ class Attention:
         self.scale = spec.scale if spec.scale is not None else spec.head_dim ** -0.5
         # the matrix-core kernels take bfloat16 with head sizes 64 and 128; every other
         # case runs the generic kernel
-        self.fast_decode = (dtype == torch.bfloat16 and
+        self.matrix_cores = (dtype == torch.bfloat16 and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
 
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self):
+        if self.matrix_cores:          # the matrix-core prefill kernel takes the same cases
+            return lib.attention_prefill_mfma_positions()
         return lib.attention_positions_per_item(self.group)
 
     def forward(self, ctx, x, entry):
@@ -94,7 +96,7 @@ class Attention:
                                     torch.float32)
                 part_ml = ctx.buffer("attn.part_ml", (n * spec.n_heads * splits * 2,),
                                      torch.float32)
-            if self.fast_decode:
+            if self.matrix_cores:
                 lib.attention_decode_mfma(q, k_pages, v_pages, meta.row_pos, meta.row_seq,
                                           page_table, out, spec.n_heads, spec.n_kv_heads,
                                           spec.head_dim, window=spec.window, scale=self.scale,
@@ -107,7 +109,14 @@ class Attention:
                               scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml)
         else:
             item_seq, item_row0, item_npos, n_items = meta.prefill_items(self.positions_per_item())
-            lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
-                          meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
-                          spec.n_kv_heads, spec.head_dim, window=spec.window, scale=self.scale)
+            if self.matrix_cores:
+                lib.attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos,
+                                           n_items, meta.row_pos, page_table, out, spec.n_heads,
+                                           spec.n_kv_heads, spec.head_dim, window=spec.window,
+                                           scale=self.scale)
+            else:
+                lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
+                              meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
+                              spec.n_kv_heads, spec.head_dim, window=spec.window,
+                              scale=self.scale)
         return self.o.forward(ctx, out, "attn.o")

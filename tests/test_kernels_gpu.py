@@ -243,8 +243,8 @@ def test_rope_small_angle_reference_vector_on_the_gpu(lib):
 
 
 # ---------------------------------------------------------------------------
-def items_for(lib, starts, counts, group):
-    per = lib.attention_positions_per_item(group)
+def items_for(lib, starts, counts, group, per=None):
+    per = per or lib.attention_positions_per_item(group)
     seq, row0, npos, row = [], [], [], 0
     for b, count in enumerate(counts):
         for p0 in range(0, count, per):
@@ -282,13 +282,18 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     pos = torch.tensor(row_pos, dtype=torch.int32, device=DEV)
     seq = torch.tensor(row_seq, dtype=torch.int32, device=DEV)
     group = nq // nkv
-    item_seq, item_row0, item_npos, n_items = items_for(lib, starts, counts, group)
+    per = lib.attention_prefill_mfma_positions() if kernel == "prefill_mfma" else None
+    item_seq, item_row0, item_npos, n_items = items_for(lib, starts, counts, group, per)
     out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=dtype)
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.full((N * nq * splits * D,), float("nan"), device=DEV)
         part_ml = torch.full((N * nq * splits * 2,), float("nan"), device=DEV)
-    if kernel == "decode_mfma":
+    if kernel == "prefill_mfma":
+        lib.attention_prefill_mfma(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0,
+                                   item_npos, n_items, pos, cache.table_dev, out, nq, nkv, D,
+                                   window=window)
+    elif kernel == "decode_mfma":
         lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
                                   cache.table_dev, out, nq, nkv, D, window=window,
                                   n_splits=splits, part_o=part_o, part_ml=part_ml)
@@ -382,6 +387,30 @@ def test_attention_decode_on_the_matrix_cores_window_and_far_key(lib, window):
         close(out, expected, torch.bfloat16)
     out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [899], [1], splits=6,
                                   boost=(0, 3, 0, 200.0), seed=4, kernel="decode_mfma")
+    close(out, expected, torch.bfloat16)
+
+
+@pytest.mark.parametrize("nq,nkv,D", [(32, 8, 128), (8, 8, 64), (6, 2, 128), (5, 1, 64)])
+def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D):
+    """The bfloat16 prefill kernel: prompts of 1, 63, 64, 65 and 300 tokens, and chunks
+    appended to 70 and to 640 cached tokens, in one launch.  Probabilities are rounded to
+    bfloat16 before the value product, which the bound (2^-8 of the largest value) covers."""
+    out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D,
+                                  starts=[0, 0, 0, 0, 70, 0, 640],
+                                  counts=[1, 64, 63, 300, 9, 65, 100], kernel="prefill_mfma")
+    close(out, expected, torch.bfloat16)
+
+
+@pytest.mark.parametrize("window", [1, 7, 64, 100])
+def test_attention_prefill_on_the_matrix_cores_window_and_far_key(lib, window):
+    nq, nkv, D, n = 8, 2, 128, 230
+    for key_index in (n - window, n - window - 1):
+        out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [0], [n], window=window,
+                                      boost=(0, key_index, n - 1, 300.0), seed=9,
+                                      kernel="prefill_mfma")
+        close(out, expected, torch.bfloat16)
+    out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [0], [900],
+                                  boost=(0, 3, 899, 200.0), seed=4, kernel="prefill_mfma")
     close(out, expected, torch.bfloat16)
 
 
