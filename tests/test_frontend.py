@@ -1,0 +1,88 @@
+"""The command line: options, chat rendering, streaming text (no GPU), and one run on a
+tiny model with a tokenizer built here (GPU)."""
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+from edge_infer_amd.frontend import chat
+from helpers import make_folder
+
+ROOT = Path(__file__).resolve().parents[1]
+
+
+def test_option_names_and_defaults_follow_the_reference():
+    """frontend/chat.py:82-96: --max_length is an alias of --max_new_tokens (424);
+    temperature 0.7, top_p 1, top_k 20."""
+    args = chat.build_parser().parse_args(["--model_path", "x"])
+    assert (args.max_new_tokens, args.temperature, args.top_p, args.top_k) == (424, 0.7, 1.0, 20)
+    assert args.model_type == "qwen3_bf16" and args.device == "cuda"
+    assert args.context_capacity is None
+    assert args.system_prompt == "You are a helpful AI assistant."
+    assert chat.build_parser().parse_args(["--model_path", "x", "--max_length", "7"]).max_new_tokens == 7
+
+
+def test_chat_rendering(tmp_path):
+    messages = [{"role": "system", "content": "S"}, {"role": "user", "content": "hi"}]
+    assert chat.render_chat(messages, tmp_path) == \
+        "<|im_start|>system\nS<|im_end|>\n<|im_start|>user\nhi<|im_end|>\n<|im_start|>assistant\n"
+    template = "{% for m in messages %}[{{ m.role }}:{{ m.content }}]{% endfor %}" \
+               "{% if add_generation_prompt %}>{% endif %}"
+    (tmp_path / "tokenizer_config.json").write_text(json.dumps({"chat_template": template}))
+    assert chat.render_chat(messages, tmp_path) == "[system:S][user:hi]>"
+
+
+def test_streaming_holds_back_incomplete_characters():
+    class Bytes:
+        """Tokens are single bytes of UTF-8 text."""
+        def decode(self, ids, skip_special_tokens=True):
+            return bytes(ids).decode("utf-8", errors="replace")
+    tok = Bytes()
+    data = list("a€b".encode("utf-8"))          # 'a', three bytes of the euro sign, 'b'
+    shown, rendered = "", ""
+    for n in range(1, len(data) + 1):
+        piece, rendered = chat.decode_stream_incremental(tok, data[:n], rendered)
+        assert "�" not in piece
+        shown += piece
+    assert shown == "a€b"
+
+
+def make_word_tokenizer(folder, vocab_size):
+    from tokenizers import Tokenizer
+    from tokenizers.models import WordLevel
+    from tokenizers.pre_tokenizers import Whitespace
+    words = ["<unk>", "<|im_start|>", "<|im_end|>", "system", "user", "assistant", "hello", "there"]
+    words += [f"w{i}" for i in range(vocab_size - len(words))]
+    tokenizer = Tokenizer(WordLevel({w: i for i, w in enumerate(words)}, unk_token="<unk>"))
+    tokenizer.pre_tokenizer = Whitespace()
+    tokenizer.save(str(folder / "tokenizer.json"))
+
+
+@pytest.mark.gpu
+def test_command_line_generates_from_ids_and_from_text(tmp_path):
+    folder = make_folder("A", tmp_path)
+    base = [sys.executable, str(ROOT / "bin" / "chat"), "--model_path", str(folder),
+            "--model_type", "qwen3_fp32", "--max_new_tokens", "6", "--temperature", "0"]
+    run = subprocess.run(base + ["--prompt_ids", "5,17,3"], capture_output=True, text=True,
+                         timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert "Total Tokens:" in run.stdout and "tokens/sec" in run.stdout
+    line = [l for l in run.stdout.split("\n") if l and l[0].isdigit()][0]
+    ids = [int(x) for x in line.split()]
+    assert 1 <= len(ids) <= 6
+    # the same tokens as the Python entry point gives
+    from edge_infer_amd.api import Model
+    session = Model.from_pretrained(folder, "qwen3_fp32").new_session(capacity=64)
+    assert session.generate([5, 17, 3], max_length=3 + 6, temperature=0.0) == ids
+    # text in, text out, with a word-level tokenizer made for this test
+    make_word_tokenizer(folder, 256)
+    run = subprocess.run(base + ["--prompt", "hello there"], capture_output=True, text=True,
+                         timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert "Total Tokens:" in run.stdout
+    # chat loop: one turn, then quit
+    run = subprocess.run(base, input="hello\nquit\n", capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stderr[-2000:]
+    assert "Assistant:" in run.stdout and "Chat started" in run.stdout
