@@ -6,9 +6,8 @@
 // lane supplies 8 consecutive k of one row, and because a dot product does not care in
 // which order k is visited, lane (row r, quarter c) takes the contiguous run
 // k0 + c*KT/4 .. + KT/4 of its row and feeds it to successive MFMAs, eight elements at a
-// time.  Each row of a 16-row tile is then read in runs of KT*2 contiguous bytes.  X (tiny)
-// is staged through LDS once per workgroup and K-tile, double-buffered, and read with the
-// same k mapping.  A workgroup is 4 waves, each owning 16 rows of W; K may be split over
+// time.  X (tiny) is staged through LDS once per workgroup and K-tile and read with the same
+// k mapping; the next tiles of W and X are already on their way while a tile is multiplied.  A workgroup is 4 waves, each owning 16 rows of W; K may be split over
 // blockIdx.y, in which case every slice writes float32 partial sums [slice, M, N] that the
 // consuming kernel adds in slice order while it reads them (deterministic, no atomics, and
 // no device-wide fence: the kernel boundary orders the writes before the reads).
@@ -20,6 +19,7 @@
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
@@ -37,7 +37,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   constexpr int CHUNKS = ROWS_X * (KT / 8);
   constexpr int XLOADS = CHUNKS / kThreads;
   static_assert(CHUNKS % kThreads == 0, "X tile must divide among the threads");
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS_X * XS];
+  __shared__ __attribute__((aligned(16))) bf16_t xs[ROWS_X * XS];
 
   const int t = threadIdx.x;
   const int wave = t / EI_WAVE, lane = t % EI_WAVE;
@@ -55,19 +55,18 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 w_cur[JN], w_next[JN];
-  uint4 x_regs[XLOADS];
-  const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
+  bf16x8 w_a[JN], w_b[JN];
+  u32x4 x_regs[XLOADS];
+  const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
 
   auto load_w = [&](bf16x8* dst, int kb) {
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
       const int k = kb + j * 32 + c * 8;
       if (k < k_end) {
-        dst[j] = *reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32);
+        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
       } else {
-        uint4 z = zero4;
-        dst[j] = *reinterpret_cast<bf16x8*>(&z);
+        dst[j] = __builtin_bit_cast(bf16x8, zero4);
       }
     }
   };
@@ -78,48 +77,54 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
       const int row = q / (KT / 8), ch = q % (KT / 8);
       const int k = kb + ch * 8;
       x_regs[i] = (row < M && k < k_end)
-                      ? *reinterpret_cast<const uint4*>(X + static_cast<size_t>(row) * K + k)
+                      ? *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(row) * K + k)
                       : zero4;
     }
   };
-  auto store_x = [&](int buf) {
+  auto store_x = [&]() {
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
       const int q = t + i * kThreads;
       const int row = q / (KT / 8), ch = q % (KT / 8);
-      *reinterpret_cast<uint4*>(&xs[buf][row * XS + ch * 8]) = x_regs[i];
+      *reinterpret_cast<u32x4*>(&xs[row * XS + ch * 8]) = x_regs[i];
     }
   };
-
-  if (n_iter > 0) {
-    load_w(w_cur, k_begin);
-    load_x(k_begin);
-    store_x(0);
-  }
-  __syncthreads();
-  for (int it = 0; it < n_iter; ++it) {
-    const int kb_next = k_begin + (it + 1) * KT;
-    const bool more = it + 1 < n_iter;
-    if (more) {
-      load_w(w_next, kb_next);
-      load_x(kb_next);
-    }
-    const bf16_t* xb = &xs[it & 1][0];
+  auto compute = [&](const bf16x8* w) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
+    for (int j = 0; j < JN; ++j) {
 #pragma unroll
-      for (int j = 0; j < JN; ++j) {
+      for (int mb = 0; mb < MB; ++mb) {
         const bf16x8 xv = *reinterpret_cast<const bf16x8*>(
-            xb + (mb * 16 + r16) * XS + j * 32 + c * 8);
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_cur[j], xv, acc[mb], 0, 0, 0);
+            &xs[(mb * 16 + r16) * XS + j * 32 + c * 8]);
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j], xv, acc[mb], 0, 0, 0);
       }
     }
-    if (more) {
-      store_x((it + 1) & 1);
-#pragma unroll
-      for (int j = 0; j < JN; ++j) w_cur[j] = w_next[j];
-    }
+  };
+  // Two register sets for W alternate, so that a tile is never copied (a copy would wait
+  // for its loads at once); the next tiles of W and X travel while this one is multiplied.
+  if (n_iter > 0) {
+    load_w(w_a, k_begin);
+    load_x(k_begin);
+  }
+  for (int it = 0; it < n_iter; it += 2) {
+    __syncthreads();                      // the previous tile of X has been read by everyone
+    store_x();
     __syncthreads();
+    if (it + 1 < n_iter) {
+      load_w(w_b, k_begin + (it + 1) * KT);
+      load_x(k_begin + (it + 1) * KT);
+    }
+    compute(w_a);
+    if (it + 1 < n_iter) {
+      __syncthreads();
+      store_x();
+      __syncthreads();
+      if (it + 2 < n_iter) {
+        load_w(w_a, k_begin + (it + 2) * KT);
+        load_x(k_begin + (it + 2) * KT);
+      }
+      compute(w_b);
+    }
   }
 
   // lane (c, r16) holds out[m = mb*16 + r16][n_tile + 4c + 0..3]
@@ -140,7 +145,93 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   }
 }
 
-int tile_for(int MB) { return MB == 4 ? 128 : 256; }
+// Up to 16 rows of X and a K range of at most kPreloadK: the whole X slice is put into LDS
+// once, after which the four waves stream their rows of W without meeting again.
+constexpr int kPreloadK = 1024;
+
+__global__ void __launch_bounds__(kThreads)
+skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
+                           float* __restrict__ out, int M, int N, int K, int k_per_split) {
+  constexpr int KT = 256, JN = KT / 32;
+  constexpr int XS = kPreloadK + 8;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * XS];
+
+  const int t = threadIdx.x;
+  const int wave = t / EI_WAVE, lane = t % EI_WAVE;
+  const int r16 = lane & 15, c = lane >> 4;
+  const int n_tile = blockIdx.x * kRowsPerBlock + wave * 16;
+  const int k_begin = blockIdx.y * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
+  const int k_len = k_end - k_begin;                 // a multiple of 8, at most kPreloadK
+  const int n_iter = (k_len + KT - 1) / KT;
+
+  // X slice -> LDS: 16 rows (zeros past M and past the slice), 16-byte chunks
+  const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
+  const int chunks_per_row = n_iter * (KT / 8);
+  for (int q = t; q < 16 * chunks_per_row; q += kThreads) {
+    const int row = q / chunks_per_row, ch = q % chunks_per_row;
+    const int k = ch * 8;
+    uint4 v = zero4;
+    if (row < M && k < k_len)
+      v = *reinterpret_cast<const uint4*>(X + static_cast<size_t>(row) * K + k_begin + k);
+    *reinterpret_cast<uint4*>(&xs[row * XS + k]) = v;
+  }
+
+  int w_row = n_tile + r16;
+  if (w_row >= N) w_row = N - 1;
+  const bf16_t* w_ptr = W + static_cast<size_t>(w_row) * K + k_begin + c * 8;
+  const bf16_t* x_ptr = &xs[r16 * XS + c * 8];
+
+  bf16x8 w_a[JN], w_b[JN];
+  auto load_w = [&](bf16x8* dst, int kb) {            // kb: offset inside the slice
+#pragma unroll
+    for (int j = 0; j < JN; ++j) {
+      if (kb + j * 32 + c * 8 < k_len) {
+        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
+      } else {
+        uint4 z = zero4;
+        dst[j] = *reinterpret_cast<bf16x8*>(&z);
+      }
+    }
+  };
+  f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
+  auto compute = [&](const bf16x8* w, int kb) {
+#pragma unroll
+    for (int j = 0; j < JN; j += 2) {
+      const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(x_ptr + kb + j * 32);
+      const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(x_ptr + kb + (j + 1) * 32);
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j], x0, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j + 1], x1, acc1, 0, 0, 0);
+    }
+  };
+  // two tiles of W in flight per wave
+  if (n_iter > 0) load_w(w_a, 0);
+  if (n_iter > 1) load_w(w_b, KT);
+  __syncthreads();
+  for (int it = 0; it < n_iter; it += 2) {
+    compute(w_a, it * KT);
+    if (it + 2 < n_iter) load_w(w_a, (it + 2) * KT);
+    if (it + 1 < n_iter) {
+      compute(w_b, (it + 1) * KT);
+      if (it + 3 < n_iter) load_w(w_b, (it + 3) * KT);
+    }
+  }
+  const f32x4 acc = acc0 + acc1;
+  float* dst = out + static_cast<size_t>(blockIdx.y) * M * N;
+  const int n0 = n_tile + 4 * c;
+  if (r16 < M) {
+    float* p = dst + static_cast<size_t>(r16) * N + n0;
+    if (n0 + 3 < N && (N & 3) == 0) {
+      *reinterpret_cast<f32x4*>(p) = acc;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (n0 + r < N) p[r] = acc[r];
+    }
+  }
+}
+
+int tile_for(int MB) { (void)MB; return 256; }
 
 }  // namespace
 
@@ -156,6 +247,11 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int target_blocks) {
   int splits = (target_blocks + row_blocks - 1) / row_blocks;
   const int max_splits = MB == 1 ? 16 : (MB == 2 ? 8 : 4);
   if (splits > max_splits) splits = max_splits;
+  if (MB == 1) {
+    // slices of at most kPreloadK let the kernel keep its X slice in LDS
+    const int need = (K + kPreloadK - 1) / kPreloadK;
+    if (splits < need && need <= 16) splits = need;
+  }
   if (splits > k_tiles) splits = k_tiles;
   if (splits < 1) splits = 1;
   const int tiles_per_split = (k_tiles + splits - 1) / splits;
@@ -185,11 +281,13 @@ extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int
   dim3 grid(row_blocks, splits);
   const bf16_t* x = static_cast<const bf16_t*>(X);
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (MB == 1)
+  if (MB == 1 && k_per_split <= kPreloadK)
+    skinny_gemm_preload_kernel<<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+  else if (MB == 1)
     skinny_gemm_kernel<1, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   else if (MB == 2)
     skinny_gemm_kernel<2, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   else
-    skinny_gemm_kernel<4, 128><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<4, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   EI_LAUNCH_CHECK();
 }

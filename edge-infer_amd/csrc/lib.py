@@ -28,6 +28,7 @@ _SIGNATURES = {
                            c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
         "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int,
                       c_void_p],
+        "ei_sum_slices": [c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
     },
     "rope_store": {
         "ei_qk_norm_rope_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_float,
@@ -184,6 +185,17 @@ def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib, status, "swiglu")
 
 
+def sum_slices(slices: torch.Tensor, out: torch.Tensor) -> None:
+    """out = slices.sum(0) for float32 [s, ...] in slice order."""
+    lib = library("rowwise")
+    n = out.numel()
+    if slices.dim() < 2 or slices[0].numel() != n:
+        raise KernelError("sum_slices: out must have the shape of one slice")
+    status = lib.ei_sum_slices(_gpu(slices, "slices", torch.float32), slices.shape[0], n,
+                               _gpu(out, "out", torch.float32), n, _stream())
+    _check(lib, status, "sum_slices")
+
+
 def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, eps, rope_table, row_pos, row_seq, page_table,
                        q_out, k_pages, v_pages, n_heads, n_kv_heads, head_dim,
                        write_cache=True) -> None:
@@ -261,12 +273,18 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
     _check(lib, status, "attention")
 
 
+MFMA_HEAD_DIMS = (64, 128)
+MFMA_PREFILL_POSITIONS = 64
+
+
 def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
-    return bool(library("attention_mfma").ei_attn_decode_mfma_supported(head_dim, group))
+    """Whether the matrix-core attention kernels take this head size (asked without
+    loading their library, so that models which do not need it never compile it)."""
+    return head_dim in MFMA_HEAD_DIMS and group >= 1
 
 
 def attention_prefill_mfma_positions() -> int:
-    return library("attention_mfma").ei_attn_prefill_mfma_positions()
+    return MFMA_PREFILL_POSITIONS
 
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,

@@ -168,7 +168,30 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
   }
 }
 
+// out[i] = sum over slices s of in[s * stride + i], in slice order.
+__global__ void sum_slices_kernel(const float* __restrict__ in, int nsplit, size_t stride,
+                                  float* __restrict__ out, size_t n) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < n; i += step) {
+    float total = in[i];
+    for (int s = 1; s < nsplit; ++s) total += in[s * stride + i];
+    out[i] = total;
+  }
+}
+
 }  // namespace
+
+extern "C" int ei_sum_slices(const float* in, int nsplit, long long stride, float* out,
+                             long long n, hipStream_t stream) {
+  EI_REQUIRE(in && out && nsplit >= 1 && n > 0 && stride >= n, "sum_slices: bad arguments");
+  const int threads = 256;
+  long long blocks = (n + threads - 1) / threads;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  sum_slices_kernel<<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
+      in, nsplit, static_cast<size_t>(stride), out, static_cast<size_t>(n));
+  EI_LAUNCH_CHECK();
+}
 
 extern "C" int ei_embed_gather(const int32_t* ids, const void* table, int table_dtype, float* out,
                                int N, int H, int V, hipStream_t stream) {

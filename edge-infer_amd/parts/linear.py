@@ -51,7 +51,15 @@ class Linear:
         if self.in_features % 8 == 0 and rows <= 4 * SKINNY_ROWS:
             for start in range(0, rows, SKINNY_ROWS):
                 stop = min(rows, start + SKINNY_ROWS)
-                lib.gemm_bf16_skinny(x[start:stop], self.weight, out[start:stop].unsqueeze(0))
+                count = stop - start
+                splits = lib.skinny_gemm_splits(count, self.out_features, self.in_features)
+                if splits == 1:
+                    lib.gemm_bf16_skinny(x[start:stop], self.weight, out[start:stop].unsqueeze(0))
+                else:
+                    slices = ctx.buffer(out_name + ".slices", (splits, count, self.out_features),
+                                        torch.float32)
+                    lib.gemm_bf16_skinny(x[start:stop], self.weight, slices)
+                    lib.sum_slices(slices, out[start:stop])
             return out
         low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)
         torch.matmul(x, self.weight.t(), out=low)

@@ -506,7 +506,7 @@ def test_gemm_bf16_skinny(lib, M, N, K):
     w = torch.randn(N, K, device=DEV).to(torch.bfloat16)
     expected = plain.linear(x.cpu(), w.cpu())
     chosen = lib.skinny_gemm_splits(M, N, K)
-    tile = 128 if M > 32 else 256
+    tile = 256
     tiles = (K + tile - 1) // tile
     candidates = {1, chosen}
     for s in range(2, tiles + 1):            # every slice count that leaves no slice empty
@@ -538,3 +538,13 @@ def test_gemm_bf16_skinny_refuses_what_it_cannot_run(lib):
     x = torch.zeros(65, 96, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(KernelError, match="1..64"):
         lib.gemm_bf16_skinny(x, w, torch.empty(1, 65, 32, device=DEV))
+
+
+def test_sum_slices(lib):
+    slices = torch.randn(5, 3, 1001, device=DEV)
+    out = torch.empty(3, 1001, device=DEV)
+    lib.sum_slices(slices, out)
+    expected = slices[0].clone()
+    for s in range(1, 5):
+        expected += slices[s]
+    assert torch.equal(out, expected)
