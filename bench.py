@@ -122,6 +122,8 @@ def main():
                         help="layers of the model (36 is the full Qwen3-8B shape)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--skip-points", action="store_true")
+    parser.add_argument("--only", choices=["decode", "prefill"], default=None,
+                        help="run one workload only and print its figures (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -134,6 +136,16 @@ def main():
     torch.cuda.synchronize()
     itemsize = 2 if args.dtype == "bfloat16" else 4
 
+    if args.only == "decode":
+        ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
+        print(json.dumps({"only": "decode", "batch": args.batch, "ms_per_step": round(ms_step, 4),
+                          "tokens_per_s": round(args.batch * 1000.0 / ms_step, 1),
+                          "context": round(context)}))
+        return 0
+    if args.only == "prefill":
+        prefill_ms = measure_prefill(model, cfg)
+        print(json.dumps({"only": "prefill", "tokens": PREFILL_TOKENS, "ms": round(prefill_ms, 3)}))
+        return 0
     ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
     value = args.batch * 1000.0 / ms_step
     achieved = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9

@@ -214,68 +214,119 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   }
 }
 
-// Prefill: a block of four waves owns 64 consecutive positions of one sequence and one query
-// head; each wave keeps 16 query rows as an MFMA operand in registers and walks the key
-// pages of the sequence.  A page of keys goes to LDS as stored, a page of values goes to LDS
-// transposed ([d][key]) so that both products read 8-element runs along their contraction
-// index.  Scores are computed transposed (S^T = K Q^T): lane (c, n) then holds, for query
-// row n, the keys 4c..4c+3 of every 16-key block, which is exactly an A-operand register
-// of P for the second product once two blocks are packed together, so the probabilities
-// never leave the registers.  Softmax state is float32; probabilities are rounded to
-// bfloat16 for the value product (the reference's prefill kernel does the same,
-// operators/src/cuda/kernels/flash_attn_prefill.cu:240).
-template <int D>
+// Prefill: a block of four waves owns HB query heads of one kv group (HB = 4, 2 or 1, the
+// largest that divides the group) and 32 * (4 / HB) consecutive positions of one sequence;
+// a wave keeps 32 rows (two 16-row tiles) of one head as MFMA operands in registers and
+// walks the key pages of the sequence.  A page of keys goes to LDS as stored, a page of
+// values goes to LDS transposed ([d][key]), once for the whole block, so the heads of a
+// group share every byte that is fetched.  Scores are computed transposed (S^T = K Q^T):
+// lane (c, n) then holds, for query row n, the keys 4c..4c+3 of every 16-key block, which is
+// exactly an A-operand register of P for the second product once two blocks are packed
+// together, so the probabilities never leave the registers.  Softmax state is float32 (in
+// units of log2); probabilities are rounded to bfloat16 for the value product (the
+// reference's prefill kernel does the same, operators/src/cuda/kernels/flash_attn_prefill.cu:240).
+// Blocks are numbered so that the blocks of one kv head fall on one XCD (the hardware deals
+// consecutive workgroups round-robin to its 8 XCDs): that head's keys and values then stay
+// in that XCD's L2.
+constexpr int kRowTiles = 2;     // 16-row tiles per wave
+
+template <int D, int HB>
 __global__ void __launch_bounds__(kThreads)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                     const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
                     const int32_t* __restrict__ item_row0, const int32_t* __restrict__ item_npos,
-                    const int32_t* __restrict__ row_pos, const int32_t* __restrict__ page_table,
-                    int table_width, bf16_t* __restrict__ out, int nq, int nkv, int window,
-                    float scale) {
+                    int n_items, const int32_t* __restrict__ row_pos,
+                    const int32_t* __restrict__ page_table, int table_width,
+                    bf16_t* __restrict__ out, int nq, int nkv, int window, float scale) {
   constexpr int DJ = D / 32;             // MFMA steps over d for the scores
   constexpr int DB = D / 16;             // 16-wide output blocks over d
   constexpr int KS = D + 8;              // LDS stride of a key row (elements)
   constexpr int VS = EI_PAGE + 8;        // LDS stride of a transposed value row
   constexpr int CI = D / 32;             // 16-byte chunks per thread per page (D/8 * 64 / 256)
+  constexpr int PW = kWaves / HB;        // waves along the positions
+  constexpr int RT = kRowTiles;
   __shared__ __attribute__((aligned(16))) bf16_t k_lds[EI_PAGE * KS];
   __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * VS];
 
-  const int item = blockIdx.x, head = blockIdx.y;
+  // block number -> (kv head, head block, item) with the kv head fixed per XCD
+  const int G = nq / nkv;
+  const int head_blocks = G / HB;
+  const int rests = n_items * head_blocks;
+  int g, rest;
+  {
+    const int id = blockIdx.x, x = id & 7, slot = id >> 3;
+    if (nkv % 8 == 0) {
+      const int per = nkv / 8;
+      g = x + 8 * (slot % per);
+      rest = slot / per;
+    } else if (8 % nkv == 0) {
+      const int share = 8 / nkv;
+      g = x % nkv;
+      rest = slot * share + x / nkv;
+    } else {
+      g = id % nkv;
+      rest = id / nkv;
+    }
+  }
+  if (rest >= rests) return;
+  const int item = rest / head_blocks, hb = rest % head_blocks;
   const int seq = item_seq[item];
   if (seq < 0) return;
   const int row0 = item_row0[item], npos = item_npos[item];
-  const int G = nq / nkv, g = head / G;
   const int t = threadIdx.x, wave = t / EI_WAVE, lane = t % EI_WAVE;
   const int r16 = lane & 15, c = lane >> 4;
+  const int hw = wave % HB, pw = wave / HB;
+  const int head = g * G + hb * HB + hw;
 
-  // this lane's query row (as column n of S^T) and its position
-  const int my_row = wave * 16 + r16;
-  const bool row_valid = my_row < npos;
-  const int pos_r = row_valid ? row_pos[row0 + my_row] : -1;
-  bf16x8 q_reg[DJ];
+  // this lane's query rows (columns n of S^T), their positions, and the Q operands
+  int pos_r[RT];
+  bool row_valid[RT];
+  bf16x8 q_reg[RT][DJ];
 #pragma unroll
-  for (int j = 0; j < DJ; ++j) {
-    uint4 z = uint4{0u, 0u, 0u, 0u};
-    if (row_valid)
-      z = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(row0 + my_row) * nq + head) * D +
-                                          j * 32 + c * 8);
-    q_reg[j] = *reinterpret_cast<bf16x8*>(&z);
+  for (int rt = 0; rt < RT; ++rt) {
+    const int my_row = pw * (16 * RT) + rt * 16 + r16;
+    row_valid[rt] = my_row < npos;
+    pos_r[rt] = row_valid[rt] ? row_pos[row0 + my_row] : -1;
+#pragma unroll
+    for (int j = 0; j < DJ; ++j) {
+      uint4 z = uint4{0u, 0u, 0u, 0u};
+      if (row_valid[rt])
+        z = *reinterpret_cast<const uint4*>(
+            q + (static_cast<size_t>(row0 + my_row) * nq + head) * D + j * 32 + c * 8);
+      q_reg[rt][j] = *reinterpret_cast<bf16x8*>(&z);
+    }
   }
 
   const int first_pos = row_pos[row0], last_pos = row_pos[row0 + npos - 1];
   const int lo_key = window > 0 ? max(0, first_pos - window + 1) : 0;
   const int lo_page = lo_key / EI_PAGE, hi_page = last_pos / EI_PAGE;
+  // the rows of this wave: pw*32 .. pw*32+31 of the item
+  const bool wave_rows_valid = pw * (16 * RT) + 16 * RT <= npos;
+  const int wave_min_pos = wave_rows_valid ? row_pos[row0 + pw * (16 * RT)] : -1;
+  const int wave_max_pos = wave_rows_valid ? row_pos[row0 + pw * (16 * RT) + 16 * RT - 1] : -1;
 
-  float m_run = kLowest, l_run = 0.f;
-  f32x4 o_acc[DB];
+  // scores are kept in units of log2 (scale * log2 e), so that 2^x is the exponential
+  const float scale_log2 = scale * 1.4426950408889634f;
+  float m_run[RT], l_run[RT];
+  f32x4 o_acc[RT][DB];
 #pragma unroll
-  for (int db = 0; db < DB; ++db) o_acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int rt = 0; rt < RT; ++rt) {
+    m_run[rt] = kLowest;
+    l_run[rt] = 0.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o_acc[rt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
 
   // global -> register staging of a page: thread t takes key t/4, chunks (t%4) + 4*i
   const int ld_key = t >> 2, ld_dc = t & 3;
   uint4 k_stage[CI], v_stage[CI];
-  auto load_page = [&](int page_index) {
-    const int phys = page_table[static_cast<size_t>(seq) * table_width + page_index];
+  // The physical page of the page after next is looked up while the next page's data is
+  // on its way, so that a page costs one trip to memory, not two in a row.
+  auto lookup = [&](int page_index) {
+    return page_index <= hi_page
+               ? page_table[static_cast<size_t>(seq) * table_width + page_index] : -1;
+  };
+  auto load_page = [&](int page_index, int phys) {
     if (phys < 0) {                       // released by the window: every key is masked
 #pragma unroll
       for (int i = 0; i < CI; ++i) k_stage[i] = v_stage[i] = uint4{0u, 0u, 0u, 0u};
@@ -306,68 +357,95 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     }
   };
 
-  load_page(lo_page);
+  load_page(lo_page, lookup(lo_page));
+  int phys_next = lookup(lo_page + 1);
   for (int page = lo_page; page <= hi_page; ++page) {
     __syncthreads();                      // the previous page's reads are done
     store_page();
     __syncthreads();
-    if (page < hi_page) load_page(page + 1);
+    if (page < hi_page) {
+      load_page(page + 1, phys_next);
+      phys_next = lookup(page + 2);
+    }
     const int key_base = page * EI_PAGE;
 
     // S^T blocks: lane (c, n) holds keys key_base + kb*16 + 4c + r for query row n
-    f32x4 s[4];
+    f32x4 s[RT][4];
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
-      s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) s[rt][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int j = 0; j < DJ; ++j) {
         const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
             &k_lds[(kb * 16 + r16) * KS + j * 32 + c * 8]);
-        s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_reg[j], s[kb], 0, 0, 0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          s[rt][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_reg[rt][j], s[rt][kb], 0, 0, 0);
       }
     }
-    float tile_max = kLowest;
+    bf16x8 p_reg[RT][2];                  // A operands of P for the two 32-key steps
+    float a_row[RT][4];
+    bool rescale = false;
+    // pages that every row of this wave sees in full (all but the last one or two of a
+    // causal prompt) need no mask
+    const bool no_mask = wave_rows_valid && key_base + EI_PAGE - 1 <= wave_min_pos &&
+                         (window <= 0 || key_base > wave_max_pos - window);
 #pragma unroll
-    for (int kb = 0; kb < 4; ++kb)
+    for (int rt = 0; rt < RT; ++rt) {
+      float tile_max = -INFINITY;
+      if (!no_mask) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int key = key_base + kb * 16 + 4 * c + r;
-        const bool visible = row_valid && key <= pos_r && (window <= 0 || key > pos_r - window);
-        const float v = visible ? s[kb][r] * scale : -INFINITY;
-        s[kb][r] = v;
-        tile_max = fmaxf(tile_max, v);
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = key_base + kb * 16 + 4 * c + r;
+            const bool visible = row_valid[rt] && key <= pos_r[rt] &&
+                                 (window <= 0 || key > pos_r[rt] - window);
+            if (!visible) s[rt][kb][r] = -INFINITY;
+          }
       }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, EI_WAVE));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, EI_WAVE));
-    const float m_new = fmaxf(m_run, tile_max);
-    const float alpha = expf(m_run - m_new);
-    float tile_sum = 0.f;
-    bf16x8 p_reg[2];                      // A operand of P for the two 32-key steps
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      bf16_t packed[8];
+      for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-      for (int half = 0; half < 2; ++half)
+        for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[rt][kb][r]);
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, EI_WAVE));
+      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, EI_WAVE));
+      // running maximum in units of log2 (raw score * scale * log2 e; the scale is positive)
+      const float m_new = fmaxf(m_run[rt], tile_max * scale_log2);
+      const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
+      float tile_sum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float p = expf(s[2 * ks + half][r] - m_new);
-          tile_sum += p;
-          packed[half * 4 + r] = ei::f32_to_bf16(p);
-        }
-      p_reg[ks] = *reinterpret_cast<bf16x8*>(packed);
+      for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[rt][2 * ks + half][r], scale_log2, -m_new));
+            tile_sum += p;
+            p_reg[rt][ks][half * 4 + r] = static_cast<__bf16>(p);
+          }
+      }
+      tile_sum += __shfl_xor(tile_sum, 16, EI_WAVE);
+      tile_sum += __shfl_xor(tile_sum, 32, EI_WAVE);
+      l_run[rt] = l_run[rt] * alpha + tile_sum;
+      m_run[rt] = m_new;
+      rescale = rescale || alpha != 1.f;
+      // the output rows of this lane are query rows 4c + r: fetch their factors
+#pragma unroll
+      for (int r = 0; r < 4; ++r) a_row[rt][r] = __shfl(alpha, 4 * c + r, EI_WAVE);
     }
-    tile_sum += __shfl_xor(tile_sum, 16, EI_WAVE);
-    tile_sum += __shfl_xor(tile_sum, 32, EI_WAVE);
-    l_run = l_run * alpha + tile_sum;
-    m_run = m_new;
-    // the output rows of this lane are query rows 4c + r: fetch their factors
-    float a_row[4];
+    const bool any_rescale = __any(rescale);
+    if (any_rescale) {                    // the maximum of some row has moved
 #pragma unroll
-    for (int r = 0; r < 4; ++r) a_row[r] = __shfl(alpha, 4 * c + r, EI_WAVE);
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) o_acc[rt][db][r] *= a_row[rt][r];
+    }
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r) o_acc[db][r] *= a_row[r];
 #pragma unroll
       for (int ks = 0; ks < 2; ++ks) {
         // values: lane (n = d column, c) supplies keys ks*32 + {4c..4c+3} and +16
@@ -375,26 +453,29 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
         const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
         const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
         uint4 both = uint4{lo.x, lo.y, hi.x, hi.y};
-        o_acc[db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-            p_reg[ks], *reinterpret_cast<bf16x8*>(&both), o_acc[db], 0, 0, 0);
+        const bf16x8 vf = *reinterpret_cast<bf16x8*>(&both);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+          o_acc[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[rt][ks], vf,
+                                                                  o_acc[rt][db], 0, 0, 0);
       }
     }
   }
 
   // lane (c, n) holds O[query row 4c + r][d = db*16 + n]
-  float inv_row[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const float l = __shfl(l_run, 4 * c + r, EI_WAVE);
-    inv_row[r] = l > 0.f ? 1.f / l : 0.f;
-  }
+  for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) {
-    const int orow = wave * 16 + 4 * c + r;
-    if (orow >= npos) continue;
-    bf16_t* dst = out + (static_cast<size_t>(row0 + orow) * nq + head) * D;
+    for (int r = 0; r < 4; ++r) {
+      const float l = __shfl(l_run[rt], 4 * c + r, EI_WAVE);
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      const int orow = pw * (16 * RT) + rt * 16 + 4 * c + r;
+      if (orow >= npos) continue;
+      bf16_t* dst = out + (static_cast<size_t>(row0 + orow) * nq + head) * D;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) dst[db * 16 + r16] = ei::from_f32<bf16_t>(o_acc[db][r] * inv_row[r]);
+      for (int db = 0; db < DB; ++db)
+        dst[db * 16 + r16] = ei::from_f32<bf16_t>(o_acc[rt][db][r] * inv);
+    }
   }
 }
 
@@ -434,10 +515,25 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
 
 }  // namespace
 
-// Positions of one sequence that a prefill work item of this file holds.
-extern "C" int ei_attn_prefill_mfma_positions() { return 64; }
+// Positions of one sequence that a prefill work item of this file holds for a group ratio.
+extern "C" int ei_attn_prefill_mfma_positions(int G) {
+  const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
+  return 16 * kRowTiles * (kWaves / HB);
+}
 
-// q, out: [N, nq, D] bfloat16; items: (sequence, first packed row, up to 64 positions).
+template <int D, int HB>
+static void launch_prefill(int blocks, hipStream_t stream, const bf16_t* q, const bf16_t* k,
+                           const bf16_t* v, const int32_t* item_seq, const int32_t* item_row0,
+                           const int32_t* item_npos, int n_items, const int32_t* row_pos,
+                           const int32_t* page_table, int table_width, bf16_t* out, int nq,
+                           int nkv, int window, float scale) {
+  attn_prefill_kernel<D, HB><<<blocks, kThreads, 0, stream>>>(
+      q, k, v, item_seq, item_row0, item_npos, n_items, row_pos, page_table, table_width, out,
+      nq, nkv, window, scale);
+}
+
+// q, out: [N, nq, D] bfloat16; items: (sequence, first packed row, positions), each holding
+// at most ei_attn_prefill_mfma_positions(nq / nkv) positions.
 extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, const void* v_pages,
                                          const int32_t* item_seq, const int32_t* item_row0,
                                          const int32_t* item_npos, int n_items,
@@ -450,20 +546,28 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
                  page_table && out && table_width > 0,
              "attention_prefill: null pointer");
   EI_REQUIRE(window >= 0, "attention_prefill: negative window");
-  EI_REQUIRE(nq <= 65535, "attention_prefill: too many heads");
-  dim3 grid(n_items, nq);
+  const int G = nq / nkv;
+  const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
+  const long long rests = static_cast<long long>(n_items) * (G / HB);
+  long long blocks;
+  if (nkv % 8 == 0) blocks = rests * nkv;
+  else if (8 % nkv == 0) blocks = (rests + 8 / nkv - 1) / (8 / nkv) * 8;
+  else blocks = rests * nkv;
+  EI_REQUIRE(blocks < (1ll << 31), "attention_prefill: too many blocks");
   const bf16_t* qq = static_cast<const bf16_t*>(q);
   const bf16_t* kk = static_cast<const bf16_t*>(k_pages);
   const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
   bf16_t* oo = static_cast<bf16_t*>(out);
-  if (D == 64)
-    attn_prefill_kernel<64><<<grid, kThreads, 0, stream>>>(qq, kk, vv, item_seq, item_row0,
-                                                           item_npos, row_pos, page_table,
-                                                           table_width, oo, nq, nkv, window, scale);
-  else
-    attn_prefill_kernel<128><<<grid, kThreads, 0, stream>>>(qq, kk, vv, item_seq, item_row0,
-                                                            item_npos, row_pos, page_table,
-                                                            table_width, oo, nq, nkv, window, scale);
+#define EI_PREFILL(DD, HH)                                                                    \
+  launch_prefill<DD, HH>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq, item_row0,   \
+                         item_npos, n_items, row_pos, page_table, table_width, oo, nq, nkv,   \
+                         window, scale)
+  if (D == 64) {
+    if (HB == 4) EI_PREFILL(64, 4); else if (HB == 2) EI_PREFILL(64, 2); else EI_PREFILL(64, 1);
+  } else {
+    if (HB == 4) EI_PREFILL(128, 4); else if (HB == 2) EI_PREFILL(128, 2); else EI_PREFILL(128, 1);
+  }
+#undef EI_PREFILL
   EI_LAUNCH_CHECK();
 }
 

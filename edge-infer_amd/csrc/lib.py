@@ -45,7 +45,7 @@ _SIGNATURES = {
     },
     "attention_mfma": {
         "ei_attn_decode_mfma_supported": [c_int, c_int],
-        "ei_attn_prefill_mfma_positions": [],
+        "ei_attn_prefill_mfma_positions": [c_int],
         "ei_attention_prefill_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
                                       c_int, c_int, c_float, c_void_p],
@@ -274,7 +274,6 @@ def attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_
 
 
 MFMA_HEAD_DIMS = (64, 128)
-MFMA_PREFILL_POSITIONS = 64
 
 
 def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
@@ -283,8 +282,11 @@ def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
     return head_dim in MFMA_HEAD_DIMS and group >= 1
 
 
-def attention_prefill_mfma_positions() -> int:
-    return MFMA_PREFILL_POSITIONS
+def attention_prefill_mfma_positions(group: int) -> int:
+    """Positions of a sequence per work item of the matrix-core prefill kernel: a block
+    holds 4, 2 or 1 heads of a kv group and 32 positions for each of its 4 waves."""
+    heads = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
+    return 32 * (4 // heads)
 
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,

@@ -87,14 +87,17 @@ class StepPlan:
                 self.items[size] = self._prefill_items(size)
 
     def _prefill_items(self, size: int):
-        item_seq, item_row0, item_npos = [], [], []
+        """(sequence, first row, positions) of every work item, the ones with the longest
+        key range first: they take longest, so they should start first."""
+        items = []
         for index, seq in enumerate(self.seqs):
             for p0 in range(0, seq.count, size):
-                item_seq.append(index)
-                item_row0.append(seq.row0 + p0)
-                item_npos.append(min(size, seq.count - p0))
-        return (np.asarray(item_seq, dtype=np.int32), np.asarray(item_row0, dtype=np.int32),
-                np.asarray(item_npos, dtype=np.int32))
+                npos = min(size, seq.count - p0)
+                items.append((-(seq.start + p0 + npos), index, seq.row0 + p0, npos))
+        items.sort()
+        return (np.asarray([i[1] for i in items], dtype=np.int32),
+                np.asarray([i[2] for i in items], dtype=np.int32),
+                np.asarray([i[3] for i in items], dtype=np.int32))
 
     def decode_items(self):
         seq = np.full(self.n_seqs, -1, dtype=np.int32)

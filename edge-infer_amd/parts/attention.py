@@ -72,7 +72,7 @@ class Attention:
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self):
         if self.matrix_cores:          # the matrix-core prefill kernel takes the same cases
-            return lib.attention_prefill_mfma_positions()
+            return lib.attention_prefill_mfma_positions(self.group)
         return lib.attention_positions_per_item(self.group)
 
     def forward(self, ctx, x, entry):

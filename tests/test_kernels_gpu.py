@@ -282,7 +282,7 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     pos = torch.tensor(row_pos, dtype=torch.int32, device=DEV)
     seq = torch.tensor(row_seq, dtype=torch.int32, device=DEV)
     group = nq // nkv
-    per = lib.attention_prefill_mfma_positions() if kernel == "prefill_mfma" else None
+    per = lib.attention_prefill_mfma_positions(group) if kernel == "prefill_mfma" else None
     item_seq, item_row0, item_npos, n_items = items_for(lib, starts, counts, group, per)
     out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=dtype)
     part_o = part_ml = None
@@ -390,7 +390,8 @@ def test_attention_decode_on_the_matrix_cores_window_and_far_key(lib, window):
     close(out, expected, torch.bfloat16)
 
 
-@pytest.mark.parametrize("nq,nkv,D", [(32, 8, 128), (8, 8, 64), (6, 2, 128), (5, 1, 64)])
+@pytest.mark.parametrize("nq,nkv,D", [(32, 8, 128), (8, 8, 64), (6, 2, 128), (5, 1, 64),
+                                      (12, 3, 128), (16, 16, 64), (8, 1, 128), (2, 1, 64)])
 def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D):
     """The bfloat16 prefill kernel: prompts of 1, 63, 64, 65 and 300 tokens, and chunks
     appended to 70 and to 640 cached tokens, in one launch.  Probabilities are rounded to
