@@ -369,31 +369,27 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     }
     const int key_base = page * EI_PAGE;
 
-    // S^T blocks: lane (c, n) holds keys key_base + kb*16 + 4c + r for query row n
-    f32x4 s[RT][4];
-#pragma unroll
-    for (int kb = 0; kb < 4; ++kb) {
-#pragma unroll
-      for (int rt = 0; rt < RT; ++rt) s[rt][kb] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < DJ; ++j) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
-            &k_lds[(kb * 16 + r16) * KS + j * 32 + c * 8]);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-          s[rt][kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_reg[rt][j], s[rt][kb], 0, 0, 0);
-      }
-    }
-    bf16x8 p_reg[RT][2];                  // A operands of P for the two 32-key steps
-    float a_row[RT][4];
-    bool rescale = false;
     // pages that every row of this wave sees in full (all but the last one or two of a
     // causal prompt) need no mask
     const bool no_mask = wave_rows_valid && key_base + EI_PAGE - 1 <= wave_min_pos &&
                          (window <= 0 || key_base > wave_max_pos - window);
+    bf16x8 p_reg[RT][2];                  // A operands of P for the two 32-key steps
+    // One row tile after the other, to keep few registers alive: scores, softmax, and
+    // (only if its maximum moved) the rescaling of that tile's output.
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
-      float tile_max = -INFINITY;
+      // S^T blocks: lane (c, n) holds keys key_base + kb*16 + 4c + r for query row n
+      f32x4 s[4];
+#pragma unroll
+      for (int kb = 0; kb < 4; ++kb) {
+        s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < DJ; ++j) {
+          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+              &k_lds[(kb * 16 + r16) * KS + j * 32 + c * 8]);
+          s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_reg[rt][j], s[kb], 0, 0, 0);
+        }
+      }
       if (!no_mask) {
 #pragma unroll
         for (int kb = 0; kb < 4; ++kb)
@@ -402,13 +398,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
             const int key = key_base + kb * 16 + 4 * c + r;
             const bool visible = row_valid[rt] && key <= pos_r[rt] &&
                                  (window <= 0 || key > pos_r[rt] - window);
-            if (!visible) s[rt][kb][r] = -INFINITY;
+            if (!visible) s[kb][r] = -INFINITY;
           }
       }
+      float tile_max = -INFINITY;
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[rt][kb][r]);
+        for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[kb][r]);
       tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, EI_WAVE));
       tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, EI_WAVE));
       // running maximum in units of log2 (raw score * scale * log2 e; the scale is positive)
@@ -421,7 +418,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
         for (int half = 0; half < 2; ++half)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[rt][2 * ks + half][r], scale_log2, -m_new));
+            const float p = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + half][r], scale_log2, -m_new));
             tile_sum += p;
             p_reg[rt][ks][half * 4 + r] = static_cast<__bf16>(p);
           }
@@ -430,19 +427,16 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       tile_sum += __shfl_xor(tile_sum, 32, EI_WAVE);
       l_run[rt] = l_run[rt] * alpha + tile_sum;
       m_run[rt] = m_new;
-      rescale = rescale || alpha != 1.f;
-      // the output rows of this lane are query rows 4c + r: fetch their factors
+      if (__any(alpha != 1.f)) {            // the maximum of some row of this tile has moved
+        // the output rows of this lane are query rows 4c + r: fetch their factors
+        float a_row[4];
 #pragma unroll
-      for (int r = 0; r < 4; ++r) a_row[rt][r] = __shfl(alpha, 4 * c + r, EI_WAVE);
-    }
-    const bool any_rescale = __any(rescale);
-    if (any_rescale) {                    // the maximum of some row has moved
+        for (int r = 0; r < 4; ++r) a_row[r] = __shfl(alpha, 4 * c + r, EI_WAVE);
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
+        for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) o_acc[rt][db][r] *= a_row[rt][r];
+          for (int r = 0; r < 4; ++r) o_acc[rt][db][r] *= a_row[r];
+      }
     }
 #pragma unroll
     for (int db = 0; db < DB; ++db) {

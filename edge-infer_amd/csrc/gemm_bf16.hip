@@ -151,7 +151,8 @@ constexpr int kPreloadK = 1024;
 
 __global__ void __launch_bounds__(kThreads)
 skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
-                           float* __restrict__ out, int M, int N, int K, int k_per_split) {
+                           float* __restrict__ out, int M, int N, int K, int k_per_split,
+                           int row_tiles) {
   constexpr int KT = 256, JN = KT / 32;
   constexpr int XS = kPreloadK + 8;
   __shared__ __attribute__((aligned(16))) bf16_t xs[16 * XS];
@@ -159,43 +160,50 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
   const int t = threadIdx.x;
   const int wave = t / EI_WAVE, lane = t % EI_WAVE;
   const int r16 = lane & 15, c = lane >> 4;
-  const int n_tile = blockIdx.x * kRowsPerBlock + wave * 16;
   const int k_begin = blockIdx.y * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
   const int k_len = k_end - k_begin;                 // a multiple of 8, at most kPreloadK
   const int n_iter = (k_len + KT - 1) / KT;
 
   // X slice -> LDS: 16 rows (zeros past M and past the slice), 16-byte chunks
-  const uint4 zero4 = uint4{0u, 0u, 0u, 0u};
+  const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
   const int chunks_per_row = n_iter * (KT / 8);
   for (int q = t; q < 16 * chunks_per_row; q += kThreads) {
     const int row = q / chunks_per_row, ch = q % chunks_per_row;
     const int k = ch * 8;
-    uint4 v = zero4;
+    u32x4 v = zero4;
     if (row < M && k < k_len)
-      v = *reinterpret_cast<const uint4*>(X + static_cast<size_t>(row) * K + k_begin + k);
-    *reinterpret_cast<uint4*>(&xs[row * XS + k]) = v;
+      v = *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(row) * K + k_begin + k);
+    *reinterpret_cast<u32x4*>(&xs[row * XS + k]) = v;
   }
-
-  int w_row = n_tile + r16;
-  if (w_row >= N) w_row = N - 1;
-  const bf16_t* w_ptr = W + static_cast<size_t>(w_row) * K + k_begin + c * 8;
   const bf16_t* x_ptr = &xs[r16 * XS + c * 8];
 
+  // The block owns `row_tiles` consecutive groups of 64 rows of W (16 per wave); the walk
+  // over (group, K-tile) is one flat pipeline with two tiles of W in flight per wave.
+  const int first_group = blockIdx.x * row_tiles;
+  const int total = row_tiles * n_iter;
+  auto w_pointer = [&](int group) {
+    int row = (first_group + group) * kRowsPerBlock + wave * 16 + r16;
+    if (row >= N) row = N - 1;                        // repeats the last row; never stored
+    return W + static_cast<size_t>(row) * K + k_begin + c * 8;
+  };
   bf16x8 w_a[JN], w_b[JN];
-  auto load_w = [&](bf16x8* dst, int kb) {            // kb: offset inside the slice
+  auto load_w = [&](bf16x8* dst, int step) {          // step = group * n_iter + tile
+    const bf16_t* w_ptr = w_pointer(step / n_iter);
+    const int kb = (step % n_iter) * KT;
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
       if (kb + j * 32 + c * 8 < k_len) {
         dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
       } else {
-        uint4 z = zero4;
-        dst[j] = *reinterpret_cast<bf16x8*>(&z);
+        dst[j] = __builtin_bit_cast(bf16x8, zero4);
       }
     }
   };
   f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
-  auto compute = [&](const bf16x8* w, int kb) {
+  float* dst = out + static_cast<size_t>(blockIdx.y) * M * N;
+  auto compute = [&](const bf16x8* w, int step) {
+    const int kb = (step % n_iter) * KT;
 #pragma unroll
     for (int j = 0; j < JN; j += 2) {
       const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(x_ptr + kb + j * 32);
@@ -203,30 +211,31 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
       acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j], x0, acc0, 0, 0, 0);
       acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j + 1], x1, acc1, 0, 0, 0);
     }
-  };
-  // two tiles of W in flight per wave
-  if (n_iter > 0) load_w(w_a, 0);
-  if (n_iter > 1) load_w(w_b, KT);
-  __syncthreads();
-  for (int it = 0; it < n_iter; it += 2) {
-    compute(w_a, it * KT);
-    if (it + 2 < n_iter) load_w(w_a, (it + 2) * KT);
-    if (it + 1 < n_iter) {
-      compute(w_b, (it + 1) * KT);
-      if (it + 3 < n_iter) load_w(w_b, (it + 3) * KT);
-    }
-  }
-  const f32x4 acc = acc0 + acc1;
-  float* dst = out + static_cast<size_t>(blockIdx.y) * M * N;
-  const int n0 = n_tile + 4 * c;
-  if (r16 < M) {
-    float* p = dst + static_cast<size_t>(r16) * N + n0;
-    if (n0 + 3 < N && (N & 3) == 0) {
-      *reinterpret_cast<f32x4*>(p) = acc;
-    } else {
+    if (step % n_iter == n_iter - 1) {                // a group of rows is complete
+      const f32x4 acc = acc0 + acc1;
+      acc0 = acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
+      const int n0 = (first_group + step / n_iter) * kRowsPerBlock + wave * 16 + 4 * c;
+      if (r16 < M) {
+        float* p = dst + static_cast<size_t>(r16) * N + n0;
+        if (n0 + 3 < N && (N & 3) == 0) {
+          *reinterpret_cast<f32x4*>(p) = acc;
+        } else {
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (n0 + r < N) p[r] = acc[r];
+          for (int r = 0; r < 4; ++r)
+            if (n0 + r < N) p[r] = acc[r];
+        }
+      }
+    }
+  };
+  if (total > 0) load_w(w_a, 0);
+  if (total > 1) load_w(w_b, 1);
+  __syncthreads();
+  for (int step = 0; step < total; step += 2) {
+    compute(w_a, step);
+    if (step + 2 < total) load_w(w_a, step + 2);
+    if (step + 1 < total) {
+      compute(w_b, step + 1);
+      if (step + 3 < total) load_w(w_b, step + 3);
     }
   }
 }
@@ -243,7 +252,7 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int target_blocks) {
   const int KT = tile_for(MB);
   const int row_blocks = (N + kRowsPerBlock - 1) / kRowsPerBlock;
   const int k_tiles = (K + KT - 1) / KT;
-  if (target_blocks <= 0) target_blocks = MB == 4 ? 512 : 1024;
+  if (target_blocks <= 0) target_blocks = 512;
   int splits = (target_blocks + row_blocks - 1) / row_blocks;
   const int max_splits = MB == 1 ? 16 : (MB == 2 ? 8 : 4);
   if (splits > max_splits) splits = max_splits;
@@ -281,8 +290,16 @@ extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int
   dim3 grid(row_blocks, splits);
   const bf16_t* x = static_cast<const bf16_t*>(X);
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (MB == 1 && k_per_split <= kPreloadK)
-    skinny_gemm_preload_kernel<<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+  if (MB == 1 && k_per_split <= kPreloadK) {
+    // fat blocks for tall matrices: several groups of 64 rows share one staged X slice,
+    // as long as some 768 blocks remain
+    int row_tiles = static_cast<int>(static_cast<long long>(row_blocks) * splits / 768);
+    if (row_tiles < 1) row_tiles = 1;
+    if (row_tiles > 8) row_tiles = 8;
+    dim3 fat((row_blocks + row_tiles - 1) / row_tiles, splits);
+    skinny_gemm_preload_kernel<<<fat, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split,
+                                                             row_tiles);
+  }
   else if (MB == 1)
     skinny_gemm_kernel<1, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   else if (MB == 2)
