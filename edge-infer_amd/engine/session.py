@@ -32,7 +32,8 @@ class _Context(StepContext):
         whose share of a short sequence is empty return at once)."""
         context = self._fixed_context or self.max_context
         pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
-        wanted = (512 + self.n_seqs * n_kv_heads - 1) // (self.n_seqs * n_kv_heads)
+        blocks = self.n_seqs * n_kv_heads
+        wanted = (512 + blocks - 1) // blocks
         return max(1, min(wanted, pages, 32))
 
 

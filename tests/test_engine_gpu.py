@@ -273,3 +273,39 @@ def test_seeded_sampling_is_the_same_alone_and_in_a_batch(folders, oracle):
     assert len({tuple(t) for t in together}) == 4
     again = session.generate_batch(prompts, first_stream=0, seed=7, **kwargs)
     assert again != together
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_one_layer_of_the_8b_shape(tmp_path, dtype):
+    """Layer sizes of Qwen3-8B (hidden 4096, 32 heads, 8 kv heads, head_dim 128,
+    intermediate 12288) with one layer and a small vocabulary: the kernels that the big
+    model uses (matrix-core attention, few-rows and library products at K = 4096 and
+    12288) against the plain implementation, whole and token by token, two sequences."""
+    import edge_infer_amd as ei
+    cfg = ei.Qwen3Config(vocab_size=1000, hidden_size=4096, num_hidden_layers=1,
+                         num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                         intermediate_size=12288, max_position_embeddings=512, bos_token_id=0,
+                         eos_token_id=999, rms_norm_eps=1e-6, rope_theta=1e6,
+                         tie_word_embeddings=False)
+    folder = ei.write_model_folder(tmp_path / "layer8b", cfg, seed=2)
+    pcfg, pw = plain.read_folder(folder)
+    a, b = random_ids(1000, 150, 5), random_ids(1000, 70, 6)
+    ref_a, ref_b = plain.forward(pw, pcfg, a), plain.forward(pw, pcfg, b)
+    model = ei.load_model(folder, dtype=dtype)
+    session = ei.Session(model, max_tokens=512, max_seqs=2)
+    sa, sb = session.begin(), session.begin()
+    logits = session.step([(sa, a[:130], list(range(130))), (sb, b[:60], list(range(60)))])
+    assert_close(dtype, logits[:130], ref_a[:130], f"8B-shape layer {dtype} prefill a")
+    assert_close(dtype, logits[130:], ref_b[:60], f"8B-shape layer {dtype} prefill b")
+    rows_a, rows_b = [], []
+    for t in range(20):
+        entries = [(sa, [a[130 + t]], [0])]
+        if t < 10:
+            entries.append((sb, [b[60 + t]], [0]))
+        out = session.step(entries)
+        rows_a.append(out[0])
+        if t < 10:
+            rows_b.append(out[1])
+    assert_close(dtype, torch.stack(rows_a), ref_a[130:], f"8B-shape layer {dtype} decode a")
+    assert_close(dtype, torch.stack(rows_b), ref_b[60:], f"8B-shape layer {dtype} decode b")
+    assert session.graph_replays > 0
