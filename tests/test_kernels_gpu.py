@@ -90,8 +90,9 @@ def test_rms_norm_reference_vector_on_the_gpu(lib):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_swiglu(lib, dtype):
-    N, I = 5, 200
+@pytest.mark.parametrize("I", [200, 100, 4096 + 8])
+def test_swiglu(lib, dtype, I):
+    N = 5
     gate_up = torch.randn(2, N, 2 * I, device=DEV) * 3
     gate_up[0, 0, 0], gate_up[1, 0, 0] = -60.0, -28.0      # the reference's -88 tail case
     out = torch.empty(N, I, device=DEV, dtype=dtype)
