@@ -482,17 +482,39 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
   const int lane = threadIdx.x % EI_WAVE;
   if (wave >= total) return;
   if (row_seq[wave / nq] < 0) return;
-  const float* ml = part_ml + static_cast<size_t>(wave) * n_splits * 2;
-  float m = kLowest;
-  for (int s = 0; s < n_splits; ++s) m = fmaxf(m, ml[2 * s]);
-  float l = 0.f;
-  for (int s = 0; s < n_splits; ++s) l += ml[2 * s + 1] * expf(ml[2 * s] - m);
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  // all slices of (m, l) and of this lane's outputs are fetched before anything is
+  // combined: one trip to memory for up to 8 slices
+  const float2* ml = reinterpret_cast<const float2*>(part_ml) + static_cast<size_t>(wave) * n_splits;
   const float* po = part_o + static_cast<size_t>(wave) * n_splits * D;
-  for (int d = lane; d < D; d += EI_WAVE) {
-    float o = 0.f;
-    for (int s = 0; s < n_splits; ++s) o += po[static_cast<size_t>(s) * D + d] * expf(ml[2 * s] - m);
-    out[static_cast<size_t>(wave) * D + d] = ei::from_f32<bf16_t>(o * inv);
+  for (int d0 = 0; d0 < D; d0 += 2 * EI_WAVE) {
+    const int d = d0 + 2 * lane;
+    float m = kLowest, l = 0.f, o0 = 0.f, o1 = 0.f;
+    for (int s0 = 0; s0 < n_splits; s0 += 8) {
+      float2 st[8], ov[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < n_splits) {
+          st[u] = ml[s0 + u];
+          ov[u] = d < D ? *reinterpret_cast<const float2*>(po + static_cast<size_t>(s0 + u) * D + d)
+                        : float2{0.f, 0.f};
+        }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (s0 + u < n_splits) {
+          const float m_new = fmaxf(m, st[u].x);
+          const float keep = expf(m - m_new), add = expf(st[u].x - m_new);
+          l = l * keep + st[u].y * add;
+          o0 = o0 * keep + ov[u].x * add;
+          o1 = o1 * keep + ov[u].y * add;
+          m = m_new;
+        }
+    }
+    if (d < D) {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      bf16_t* dst = out + static_cast<size_t>(wave) * D + d;
+      dst[0] = ei::from_f32<bf16_t>(o0 * inv);
+      dst[1] = ei::from_f32<bf16_t>(o1 * inv);
+    }
   }
 }
 

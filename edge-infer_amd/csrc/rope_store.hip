@@ -47,9 +47,21 @@ __global__ void qk_norm_rope_store_kernel(
     x[j] = 0.f;
     y[j] = 0.f;
     if (i < half) {
-      for (int s = 0; s < nsplit; ++s) {
-        x[j] += ei::to_f32<TI>(src[s * split_stride + i]);
-        y[j] += ei::to_f32<TI>(src[s * split_stride + i + half]);
+      // slices are added in slice order, four loads per trip to memory
+      for (int s0 = 0; s0 < nsplit; s0 += 4) {
+        TI a[4], b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (s0 + u < nsplit) {
+            a[u] = src[(s0 + u) * split_stride + i];
+            b[u] = src[(s0 + u) * split_stride + i + half];
+          }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          if (s0 + u < nsplit) {
+            x[j] += ei::to_f32<TI>(a[u]);
+            y[j] += ei::to_f32<TI>(b[u]);
+          }
       }
       sum += x[j] * x[j] + y[j] * y[j];
     }

@@ -113,21 +113,19 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
       Vec4<float>::load(res + qd * 4, x[k]);
       if (HAS_DELTA) {
         const TD* d = delta + static_cast<size_t>(src) * H + qd * 4;
-        int s = 0;
-        for (; s + 4 <= nsplit; s += 4) {       // four independent loads in flight
-          float a[4], b[4], c[4], e[4];
-          Vec4<TD>::load(d + (s + 0) * split_stride, a);
-          Vec4<TD>::load(d + (s + 1) * split_stride, b);
-          Vec4<TD>::load(d + (s + 2) * split_stride, c);
-          Vec4<TD>::load(d + (s + 3) * split_stride, e);
+        // slices are added in slice order; eight loads are issued before the first sum so
+        // that a row costs one trip to memory per eight slices
+        for (int s0 = 0; s0 < nsplit; s0 += 8) {
+          float v[8][4];
 #pragma unroll
-          for (int i = 0; i < 4; ++i) x[k][i] = (((x[k][i] + a[i]) + b[i]) + c[i]) + e[i];
-        }
-        for (; s < nsplit; ++s) {
-          float a[4];
-          Vec4<TD>::load(d + s * split_stride, a);
+          for (int u = 0; u < 8; ++u)
+            if (s0 + u < nsplit) Vec4<TD>::load(d + (s0 + u) * split_stride, v[u]);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) x[k][i] += a[i];
+          for (int u = 0; u < 8; ++u)
+            if (s0 + u < nsplit) {
+#pragma unroll
+              for (int i = 0; i < 4; ++i) x[k][i] += v[u][i];
+            }
         }
         if (write_residual) Vec4<float>::store(res + qd * 4, x[k]);
       }
@@ -135,16 +133,21 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
       for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
     }
   }
+  float w[CHUNKS][4];                      // fetched before the reduction, not after it
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) Vec4<float>::load(weight + qd * 4, w[k]);
+  }
   const float total = ei::block_sum(sum, scratch);
   const float inv = rsqrtf(total / static_cast<float>(H) + eps);
 #pragma unroll
   for (int k = 0; k < CHUNKS; ++k) {
     const int qd = threadIdx.x + k * blockDim.x;
     if (qd < quads) {
-      float w[4], y[4];
-      Vec4<float>::load(weight + qd * 4, w);
+      float y[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) y[i] = (x[k][i] * inv) * w[i];
+      for (int i = 0; i < 4; ++i) y[i] = (x[k][i] * inv) * w[k][i];
       Vec4<TO>::store(dst + qd * 4, y);
     }
   }
@@ -183,19 +186,28 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
     float gate[8], up[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) gate[i] = up[i] = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-      float a[4], b[4], c[4], d[4];
-      Vec4<TI>::load(g + s * split_stride, a);
-      Vec4<TI>::load(g + s * split_stride + 4, b);
-      Vec4<TI>::load(g + s * split_stride + I, c);
-      Vec4<TI>::load(g + s * split_stride + I + 4, d);
+    for (int s0 = 0; s0 < nsplit; s0 += 4) {     // four slices per trip to memory
+      float a[4][4], b[4][4], c[4][4], d[4][4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        gate[i] += a[i];
-        gate[i + 4] += b[i];
-        up[i] += c[i];
-        up[i + 4] += d[i];
-      }
+      for (int u = 0; u < 4; ++u)
+        if (s0 + u < nsplit) {
+          const TI* p = g + (s0 + u) * split_stride;
+          Vec4<TI>::load(p, a[u]);
+          Vec4<TI>::load(p + 4, b[u]);
+          Vec4<TI>::load(p + I, c[u]);
+          Vec4<TI>::load(p + I + 4, d[u]);
+        }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (s0 + u < nsplit) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            gate[i] += a[u][i];
+            gate[i + 4] += b[u][i];
+            up[i] += c[u][i];
+            up[i + 4] += d[u][i];
+          }
+        }
     }
     float y0[4], y1[4];
 #pragma unroll
