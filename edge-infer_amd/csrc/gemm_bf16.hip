@@ -26,8 +26,15 @@ namespace {
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * EI_WAVE;
 constexpr int kRowsPerBlock = kWaves * 16;
+constexpr int kPackedTile = 16 * 32;      // elements of one packed tile: 16 rows x 32 k, 1 KB
 
-template <int MB, int KT>
+// Address of the 16-byte piece that lane `lane` takes of the packed tile (kt, strip).
+__device__ __forceinline__ const bf16_t* packed_piece(const bf16_t* Wp, int n_strips, int kt,
+                                                      int strip, int lane) {
+  return Wp + (static_cast<size_t>(kt) * n_strips + strip) * kPackedTile + lane * 8;
+}
+
+template <int MB, int KT, bool PACKED>
 __global__ void __launch_bounds__(kThreads)
 skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
                    float* __restrict__ out, int M, int N, int K, int k_per_split) {
@@ -49,7 +56,11 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
 
   int w_row = n_tile + r16;
   if (w_row >= N) w_row = N - 1;          // rows past the end repeat the last one; never stored
-  const bf16_t* w_ptr = W + static_cast<size_t>(w_row) * K + c * 8;
+  const int n_strips = (N + 15) / 16;
+  const int strip = min(n_tile / 16, n_strips - 1);
+  const bf16_t* w_ptr = PACKED ? packed_piece(W, n_strips, 0, strip, lane)
+                               : W + static_cast<size_t>(w_row) * K + c * 8;
+  const size_t tile_stride = static_cast<size_t>(n_strips) * kPackedTile;
 
   f32x4 acc[MB];
 #pragma unroll
@@ -62,9 +73,10 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   auto load_w = [&](bf16x8* dst, int kb) {
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
-      const int k = kb + j * 32 + c * 8;
+      const int k = kb + j * 32 + (PACKED ? 0 : c * 8);   // packed tiles are zero past K
       if (k < k_end) {
-        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
+        const bf16_t* src = PACKED ? w_ptr + (kb / 32 + j) * tile_stride : w_ptr + kb + j * 32;
+        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src));
       } else {
         dst[j] = __builtin_bit_cast(bf16x8, zero4);
       }
@@ -149,6 +161,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
 // once, after which the four waves stream their rows of W without meeting again.
 constexpr int kPreloadK = 1024;
 
+template <bool PACKED>
 __global__ void __launch_bounds__(kThreads)
 skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
                            float* __restrict__ out, int M, int N, int K, int k_per_split,
@@ -182,7 +195,13 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
   // over (group, K-tile) is one flat pipeline with two tiles of W in flight per wave.
   const int first_group = blockIdx.x * row_tiles;
   const int total = row_tiles * n_iter;
+  const int n_strips = (N + 15) / 16;
+  const size_t tile_stride = static_cast<size_t>(n_strips) * kPackedTile;
   auto w_pointer = [&](int group) {
+    if (PACKED) {
+      const int strip = min((first_group + group) * kWaves + wave, n_strips - 1);
+      return packed_piece(W, n_strips, k_begin / 32, strip, lane);
+    }
     int row = (first_group + group) * kRowsPerBlock + wave * 16 + r16;
     if (row >= N) row = N - 1;                        // repeats the last row; never stored
     return W + static_cast<size_t>(row) * K + k_begin + c * 8;
@@ -193,8 +212,9 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
     const int kb = (step % n_iter) * KT;
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
-      if (kb + j * 32 + c * 8 < k_len) {
-        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
+      if (kb + j * 32 + (PACKED ? 0 : c * 8) < k_len) {
+        const bf16_t* src = PACKED ? w_ptr + (kb / 32 + j) * tile_stride : w_ptr + kb + j * 32;
+        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src));
       } else {
         dst[j] = __builtin_bit_cast(bf16x8, zero4);
       }
@@ -269,8 +289,11 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int target_blocks) {
 
 // X: [M, K] bfloat16, W: [N, K] bfloat16, out: [splits, M, N] float32 (slice s holds the
 // sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 64.
-extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int M, int N, int K,
-                                   int splits, hipStream_t stream) {
+namespace {
+
+template <bool PACKED>
+int launch_skinny(const void* X, const void* W, float* out, int M, int N, int K, int splits,
+                  hipStream_t stream) {
   EI_REQUIRE(M >= 1 && M <= 64, "gemm_bf16_skinny: rows must lie in 1..64");
   EI_REQUIRE(N >= 1 && K >= 8 && K % 8 == 0, "gemm_bf16_skinny: K must be a multiple of 8");
   EI_REQUIRE(X && W && out, "gemm_bf16_skinny: null pointer");
@@ -297,14 +320,34 @@ extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int
     if (row_tiles < 1) row_tiles = 1;
     if (row_tiles > 8) row_tiles = 8;
     dim3 fat((row_blocks + row_tiles - 1) / row_tiles, splits);
-    skinny_gemm_preload_kernel<<<fat, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split,
-                                                             row_tiles);
+    skinny_gemm_preload_kernel<PACKED><<<fat, kThreads, 0, stream>>>(w, x, out, M, N, K,
+                                                                     k_per_split, row_tiles);
   }
   else if (MB == 1)
-    skinny_gemm_kernel<1, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<1, 256, PACKED><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   else if (MB == 2)
-    skinny_gemm_kernel<2, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<2, 256, PACKED><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   else
-    skinny_gemm_kernel<4, 256><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<4, 256, PACKED><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   EI_LAUNCH_CHECK();
+}
+
+}  // namespace
+
+// X: [M, K] bfloat16, W: [N, K] bfloat16, out: [splits, M, N] float32 (slice s holds the
+// sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 64.
+extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int M, int N, int K,
+                                   int splits, hipStream_t stream) {
+  return launch_skinny<false>(X, W, out, M, N, K, splits, stream);
+}
+
+// The same product with W in the streaming layout: tiles of 16 rows x 32 k (1 KB each, rows
+// past N and k past K zero), tile (kt, strip) at index kt * ceil(N/16) + strip, and inside a
+// tile the piece of lane (c = k/8 % 4, r = row % 16) at (c * 16 + r) * 8 elements, i.e. the
+// order in which a wave's lanes hold an MFMA operand.  A wave's load is then one contiguous
+// kilobyte and the waves that run together read neighbouring kilobytes, which keeps every
+// memory channel busy; rows of W that are 2^n bytes apart do not.
+extern "C" int ei_gemm_bf16_skinny_packed(const void* X, const void* Wp, float* out, int M, int N,
+                                          int K, int splits, hipStream_t stream) {
+  return launch_skinny<true>(X, Wp, out, M, N, K, splits, stream);
 }

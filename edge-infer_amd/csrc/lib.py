@@ -61,6 +61,8 @@ _SIGNATURES = {
         "ei_skinny_gemm_splits": [c_int, c_int, c_int, c_int],
         "ei_gemm_bf16_skinny": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                 c_void_p],
+        "ei_gemm_bf16_skinny_packed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                       c_void_p],
     },
     "sampling": {
         "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
@@ -416,3 +418,35 @@ def gemm_bf16_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Non
                                      _gpu(out, "out", torch.float32), m, n, k, out.shape[0],
                                      _stream())
     _check(lib, status, "gemm_bf16_skinny")
+
+
+def pack_weight(w: torch.Tensor) -> torch.Tensor:
+    """The streaming copy of a bfloat16 matrix [n, k] for `gemm_bf16_skinny_packed`:
+    [ceil(k/32), ceil(n/16), 4, 16, 8] where element (kt, strip, c, r, e) is
+    w[strip*16 + r, kt*32 + c*8 + e], zero outside the matrix.  Made once when the weights
+    are loaded; a data movement, no arithmetic."""
+    if w.dtype != torch.bfloat16 or w.dim() != 2:
+        raise KernelError("pack_weight: a bfloat16 matrix is expected")
+    n, k = w.shape
+    strips, tiles = (n + 15) // 16, (k + 31) // 32
+    if (strips * 16, tiles * 32) != (n, k):
+        padded = torch.zeros((strips * 16, tiles * 32), dtype=w.dtype, device=w.device)
+        padded[:n, :k] = w
+        w = padded
+    return w.view(strips, 16, tiles, 4, 8).permute(2, 0, 3, 1, 4).contiguous()
+
+
+def gemm_bf16_skinny_packed(x: torch.Tensor, packed: torch.Tensor, n: int,
+                            out: torch.Tensor) -> None:
+    """`gemm_bf16_skinny` with the weight given as `pack_weight(w)` of a matrix [n, k]."""
+    lib = library("gemm_bf16")
+    m, k = x.shape
+    if (out.dim() != 3 or tuple(out.shape[1:]) != (m, n) or packed.dim() != 5
+            or tuple(packed.shape) != ((k + 31) // 32, (n + 15) // 16, 4, 16, 8)):
+        raise KernelError(f"gemm_bf16_skinny_packed: shapes {list(x.shape)} x packed "
+                          f"{list(packed.shape)} (n = {n}) -> {list(out.shape)} do not agree")
+    status = lib.ei_gemm_bf16_skinny_packed(_gpu(x, "x", torch.bfloat16),
+                                            _gpu(packed, "packed", torch.bfloat16),
+                                            _gpu(out, "out", torch.float32), m, n, k,
+                                            out.shape[0], _stream())
+    _check(lib, status, "gemm_bf16_skinny_packed")

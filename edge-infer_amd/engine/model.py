@@ -80,11 +80,8 @@ class DecoderModel:
                                     self.device)
         if "head.weight" in params and params["head.weight"] is not params["embed.weight"]:
             self.head = Linear(params["head.weight"], self.dtype, self.device)
-        else:  # tied: the head is the embedding table itself
-            self.head = Linear.__new__(Linear)
-            self.head.weight = self.embed
-            self.head.out_features, self.head.in_features = self.embed.shape
-            self.head.dtype = self.dtype
+        else:  # tied: the head is the embedding table itself (no copy: same type and device)
+            self.head = Linear(self.embed, self.dtype, self.device)
 
     def position_table(self, position_spec):
         """One shared encoding object per distinct position spec."""

@@ -5,14 +5,24 @@ bfloat16: for up to `SKINNY_ROWS` rows the hand-written weight-streaming MFMA
 kernel, which returns float32 partial sums [slices, rows, out] that the consuming
 kernel adds up while it reads them; for more rows the library matrix product (the reference multiplies
 through cuBLAS as well, operators/src/cuda/execution.cu:299-324).
+
+The few-rows kernel reads a second copy of the weight in its streaming layout (tiles in
+the order in which the matrix cores take them, see `lib.pack_weight`), made when the
+weight is loaded: decode is bound by how fast the weights can be read, and the
+contiguous copy reads about a fifth faster than rows that lie a power of two apart.  It
+doubles the memory of the linear weights; EDGE_INFER_STREAM_COPY=0 keeps only the stored
+layout and lets the kernel read that.
 """
 from __future__ import annotations
+
+import os
 
 import torch
 
 from ..csrc import lib
 
 SKINNY_ROWS = 64
+STREAM_COPY = os.environ.get("EDGE_INFER_STREAM_COPY", "1") != "0"
 
 
 class Linear:
@@ -22,6 +32,15 @@ class Linear:
         self.weight = weight.to(device=device, dtype=dtype).contiguous()
         self.out_features, self.in_features = self.weight.shape
         self.dtype = dtype
+        self.packed = None
+        if dtype == torch.bfloat16 and STREAM_COPY and self.in_features % 8 == 0:
+            self.packed = lib.pack_weight(self.weight)
+
+    def _few_rows(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        if self.packed is not None:
+            lib.gemm_bf16_skinny_packed(x, self.packed, self.out_features, out)
+        else:
+            lib.gemm_bf16_skinny(x, self.weight, out)
 
     def forward(self, ctx, x: torch.Tensor, out_name: str) -> torch.Tensor:
         """x [N, in] of the step's storage type -> [N, out] in the storage type, or float32
@@ -35,7 +54,7 @@ class Linear:
         if lib.skinny_gemm_ok(rows, self.in_features):
             splits = lib.skinny_gemm_splits(rows, self.out_features, self.in_features)
             out = ctx.buffer(out_name + ".f32", (splits, rows, self.out_features), torch.float32)
-            lib.gemm_bf16_skinny(x, self.weight, out)
+            self._few_rows(x, out)
             return out
         out = ctx.buffer(out_name, (rows, self.out_features), torch.bfloat16)
         torch.matmul(x, self.weight.t(), out=out)
@@ -54,11 +73,11 @@ class Linear:
                 count = stop - start
                 splits = lib.skinny_gemm_splits(count, self.out_features, self.in_features)
                 if splits == 1:
-                    lib.gemm_bf16_skinny(x[start:stop], self.weight, out[start:stop].unsqueeze(0))
+                    self._few_rows(x[start:stop], out[start:stop].unsqueeze(0))
                 else:
                     slices = ctx.buffer(out_name + ".slices", (splits, count, self.out_features),
                                         torch.float32)
-                    lib.gemm_bf16_skinny(x[start:stop], self.weight, slices)
+                    self._few_rows(x[start:stop], slices)
                     lib.sum_slices(slices, out[start:stop])
             return out
         low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)

@@ -516,12 +516,18 @@ def test_gemm_bf16_skinny(lib, M, N, K):
         if (tiles + per - 1) // per == s:
             candidates.add(s)
     results = {}
+    packed = lib.pack_weight(w)
+    assert packed.shape == ((K + 31) // 32, (N + 15) // 16, 4, 16, 8)
     for splits in sorted(candidates):
         out = torch.full((splits, M, N), float("nan"), device=DEV)
         lib.gemm_bf16_skinny(x, w, out)
         err = (out.double().cpu().sum(0) - expected).abs().max().item()
         assert err <= 2e-6 * math.sqrt(K) * 16, f"splits {splits}: max error {err:.3e}"
         results[splits] = out
+        # the streaming copy of the weight: the same sums in the same order
+        again = torch.full((splits, M, N), float("nan"), device=DEV)
+        lib.gemm_bf16_skinny_packed(x, packed, N, again)
+        assert torch.equal(again, out), f"splits {splits}: packed layout differs"
     # a row gives the same bits alone as inside a batch of up to 16 rows (the same tile
     # shape and slice count, hence the same order of accumulation)
     if M <= 16 and lib.skinny_gemm_splits(1, N, K) == chosen:
@@ -540,6 +546,8 @@ def test_gemm_bf16_skinny_refuses_what_it_cannot_run(lib):
     x = torch.zeros(65, 96, device=DEV, dtype=torch.bfloat16)
     with pytest.raises(KernelError, match="1..64"):
         lib.gemm_bf16_skinny(x, w, torch.empty(1, 65, 32, device=DEV))
+    with pytest.raises(KernelError, match="do not agree"):       # packed for another n
+        lib.gemm_bf16_skinny_packed(x[:2], lib.pack_weight(w), 48, torch.empty(1, 2, 48, device=DEV))
 
 
 def test_sum_slices(lib):
