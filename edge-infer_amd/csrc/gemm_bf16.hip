@@ -73,10 +73,16 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   auto load_w = [&](bf16x8* dst, int kb) {
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
-      const int k = kb + j * 32 + (PACKED ? 0 : c * 8);   // packed tiles are zero past K
+      if (PACKED) {
+        // the packed copy holds whole K-tiles (zeros past K): no test, so that the loads
+        // form one straight run whose arrival the compiler can count
+        dst[j] = __builtin_nontemporal_load(
+            reinterpret_cast<const bf16x8*>(w_ptr + (kb / 32 + j) * tile_stride));
+        continue;
+      }
+      const int k = kb + j * 32 + c * 8;
       if (k < k_end) {
-        const bf16_t* src = PACKED ? w_ptr + (kb / 32 + j) * tile_stride : w_ptr + kb + j * 32;
-        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src));
+        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
       } else {
         dst[j] = __builtin_bit_cast(bf16x8, zero4);
       }
@@ -178,17 +184,29 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
   const int k_len = k_end - k_begin;                 // a multiple of 8, at most kPreloadK
   const int n_iter = (k_len + KT - 1) / KT;
 
-  // X slice -> LDS: 16 rows (zeros past M and past the slice), 16-byte chunks
+  // X slice -> LDS: 16 rows (zeros past M and past the slice), 16-byte chunks, at most 8
+  // per thread.  Every load is issued (from a clamped address) before the first is used.
   const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
   const int chunks_per_row = n_iter * (KT / 8);
-  for (int q = t; q < 16 * chunks_per_row; q += kThreads) {
-    const int row = q / chunks_per_row, ch = q % chunks_per_row;
-    const int k = ch * 8;
-    u32x4 v = zero4;
-    if (row < M && k < k_len)
-      v = *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(row) * K + k_begin + k);
-    *reinterpret_cast<u32x4*>(&xs[row * XS + k]) = v;
+  constexpr int XCH = 16 * (kPreloadK / 8) / kThreads;
+  u32x4 xv[XCH];
+#pragma unroll
+  for (int i = 0; i < XCH; ++i) {
+    const int q = t + i * kThreads;
+    const int row = q / chunks_per_row, k = (q % chunks_per_row) * 8;
+    const bool valid = row < M && k < k_len;
+    const u32x4 v = *reinterpret_cast<const u32x4*>(
+        X + static_cast<size_t>(valid ? row : 0) * K + k_begin + (valid ? k : 0));
+    xv[i] = valid ? v : zero4;
   }
+  auto store_x = [&]() {                               // after the first loads of W are issued
+#pragma unroll
+    for (int i = 0; i < XCH; ++i) {
+      const int q = t + i * kThreads;
+      const int row = q / chunks_per_row, k = (q % chunks_per_row) * 8;
+      if (row < 16) *reinterpret_cast<u32x4*>(&xs[row * XS + k]) = xv[i];
+    }
+  };
   const bf16_t* x_ptr = &xs[r16 * XS + c * 8];
 
   // The block owns `row_tiles` consecutive groups of 64 rows of W (16 per wave); the walk
@@ -212,9 +230,13 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
     const int kb = (step % n_iter) * KT;
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
-      if (kb + j * 32 + (PACKED ? 0 : c * 8) < k_len) {
-        const bf16_t* src = PACKED ? w_ptr + (kb / 32 + j) * tile_stride : w_ptr + kb + j * 32;
-        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(src));
+      if (PACKED) {
+        dst[j] = __builtin_nontemporal_load(
+            reinterpret_cast<const bf16x8*>(w_ptr + (kb / 32 + j) * tile_stride));
+        continue;
+      }
+      if (kb + j * 32 + c * 8 < k_len) {
+        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
       } else {
         dst[j] = __builtin_bit_cast(bf16x8, zero4);
       }
@@ -247,16 +269,34 @@ skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restric
       }
     }
   };
-  if (total > 0) load_w(w_a, 0);
-  if (total > 1) load_w(w_b, 1);
+  // The loads of the steady loop are unconditional, so that on every path into a product
+  // the same number of loads is outstanding and the wait before it can let the younger
+  // tile stay in flight; the last two or three steps are peeled off.
+  if (total == 1) {
+    load_w(w_a, 0);
+    store_x();
+    __syncthreads();
+    compute(w_a, 0);
+    return;
+  }
+  load_w(w_a, 0);
+  load_w(w_b, 1);
+  store_x();
   __syncthreads();
-  for (int step = 0; step < total; step += 2) {
+  int step = 0;
+  for (; step + 3 < total; step += 2) {
     compute(w_a, step);
-    if (step + 2 < total) load_w(w_a, step + 2);
-    if (step + 1 < total) {
-      compute(w_b, step + 1);
-      if (step + 3 < total) load_w(w_b, step + 3);
-    }
+    load_w(w_a, step + 2);
+    compute(w_b, step + 1);
+    load_w(w_b, step + 3);
+  }
+  compute(w_a, step);
+  if (step + 2 < total) {
+    load_w(w_a, step + 2);
+    compute(w_b, step + 1);
+    compute(w_a, step + 2);
+  } else {
+    compute(w_b, step + 1);
   }
 }
 
@@ -342,7 +382,8 @@ extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int
 }
 
 // The same product with W in the streaming layout: tiles of 16 rows x 32 k (1 KB each, rows
-// past N and k past K zero), tile (kt, strip) at index kt * ceil(N/16) + strip, and inside a
+// past N and k past K zero, K padded to a multiple of 256 so that every K-tile of the kernel
+// is whole), tile (kt, strip) at index kt * ceil(N/16) + strip, and inside a
 // tile the piece of lane (c = k/8 % 4, r = row % 16) at (c * 16 + r) * 8 elements, i.e. the
 // order in which a wave's lanes hold an MFMA operand.  A wave's load is then one contiguous
 // kilobyte and the waves that run together read neighbouring kilobytes, which keeps every

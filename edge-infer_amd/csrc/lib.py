@@ -422,13 +422,14 @@ def gemm_bf16_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> Non
 
 def pack_weight(w: torch.Tensor) -> torch.Tensor:
     """The streaming copy of a bfloat16 matrix [n, k] for `gemm_bf16_skinny_packed`:
-    [ceil(k/32), ceil(n/16), 4, 16, 8] where element (kt, strip, c, r, e) is
-    w[strip*16 + r, kt*32 + c*8 + e], zero outside the matrix.  Made once when the weights
+    [8*ceil(k/256), ceil(n/16), 4, 16, 8] where element (kt, strip, c, r, e) is
+    w[strip*16 + r, kt*32 + c*8 + e], zero outside the matrix (k is padded to whole
+    K-tiles of the kernel, 256 wide).  Made once when the weights
     are loaded; a data movement, no arithmetic."""
     if w.dtype != torch.bfloat16 or w.dim() != 2:
         raise KernelError("pack_weight: a bfloat16 matrix is expected")
     n, k = w.shape
-    strips, tiles = (n + 15) // 16, (k + 31) // 32
+    strips, tiles = (n + 15) // 16, 8 * ((k + 255) // 256)
     if (strips * 16, tiles * 32) != (n, k):
         padded = torch.zeros((strips * 16, tiles * 32), dtype=w.dtype, device=w.device)
         padded[:n, :k] = w
@@ -442,7 +443,7 @@ def gemm_bf16_skinny_packed(x: torch.Tensor, packed: torch.Tensor, n: int,
     lib = library("gemm_bf16")
     m, k = x.shape
     if (out.dim() != 3 or tuple(out.shape[1:]) != (m, n) or packed.dim() != 5
-            or tuple(packed.shape) != ((k + 31) // 32, (n + 15) // 16, 4, 16, 8)):
+            or tuple(packed.shape) != (8 * ((k + 255) // 256), (n + 15) // 16, 4, 16, 8)):
         raise KernelError(f"gemm_bf16_skinny_packed: shapes {list(x.shape)} x packed "
                           f"{list(packed.shape)} (n = {n}) -> {list(out.shape)} do not agree")
     status = lib.ei_gemm_bf16_skinny_packed(_gpu(x, "x", torch.bfloat16),

@@ -517,7 +517,7 @@ def test_gemm_bf16_skinny(lib, M, N, K):
             candidates.add(s)
     results = {}
     packed = lib.pack_weight(w)
-    assert packed.shape == ((K + 31) // 32, (N + 15) // 16, 4, 16, 8)
+    assert packed.shape == (8 * ((K + 255) // 256), (N + 15) // 16, 4, 16, 8)
     for splits in sorted(candidates):
         out = torch.full((splits, M, N), float("nan"), device=DEV)
         lib.gemm_bf16_skinny(x, w, out)
