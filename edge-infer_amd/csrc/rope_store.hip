@@ -108,6 +108,111 @@ __global__ void qk_norm_rope_store_kernel(
   }
 }
 
+// The same for head sizes that are a multiple of 8: G lanes (a power of two) share a head,
+// each lane takes 4 neighbouring pairs with one 8- or 16-byte access per half, so a wave
+// covers 64 / G heads.
+template <typename TI, typename TO, int G>
+__global__ void qk_norm_rope_store_vec_kernel(
+    const TI* __restrict__ qkv, int nsplit, size_t split_stride,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ rope_table, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
+    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
+    int N, int nq, int nkv, int D, int write_cache) {
+  using ei::Vec4;
+  const int heads = nq + 2 * nkv;
+  const long long item = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) / G;
+  const int sub = threadIdx.x % G;
+  if (item >= static_cast<long long>(N) * heads) return;       // the same for all lanes of a group
+  const int row = static_cast<int>(item / heads), head = static_cast<int>(item % heads);
+  const int seq = row_seq[row];
+  if (seq < 0) return;  // padding row
+  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  if (!is_q && !write_cache) return;
+  const int pos = row_pos[row];
+  const int half = D / 2;
+  const int i0 = sub * 4;
+  const bool active = i0 < half;
+  const size_t width = static_cast<size_t>(heads) * D;
+  const TI* src = qkv + static_cast<size_t>(row) * width + static_cast<size_t>(head) * D + i0;
+
+  TO* dst;
+  bool stored = true;
+  if (is_q) {
+    dst = q_out + static_cast<size_t>(row) * nq * D + static_cast<size_t>(head) * D;
+  } else {
+    const int page = page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE];
+    stored = page >= 0;
+    const int g = is_k ? head - nq : head - nq - nkv;
+    TO* base = is_k ? k_pages : v_pages;
+    dst = base + ((static_cast<size_t>(stored ? page : 0) * nkv + g) * EI_PAGE + pos % EI_PAGE) * D;
+  }
+  const float* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
+  const bool rotate = rope_table != nullptr && (is_q || is_k);
+
+  float x[4] = {0.f, 0.f, 0.f, 0.f}, y[4] = {0.f, 0.f, 0.f, 0.f};
+  float wx[4] = {1.f, 1.f, 1.f, 1.f}, wy[4] = {1.f, 1.f, 1.f, 1.f};
+  float cs[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
+  if (active) {
+    for (int s0 = 0; s0 < nsplit; s0 += 4) {       // slices in slice order, four per trip
+      float a[4][4], b[4][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (s0 + u < nsplit) {
+          Vec4<TI>::load(src + (s0 + u) * split_stride, a[u]);
+          Vec4<TI>::load(src + (s0 + u) * split_stride + half, b[u]);
+        }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (s0 + u < nsplit) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            x[i] += a[u][i];
+            y[i] += b[u][i];
+          }
+        }
+    }
+    if (norm_w) {
+      Vec4<float>::load(norm_w + i0, wx);
+      Vec4<float>::load(norm_w + i0 + half, wy);
+    }
+    if (rotate) {
+      const float* trig = rope_table + static_cast<size_t>(pos) * D + i0;
+      Vec4<float>::load(trig, cs);
+      Vec4<float>::load(trig + half, sn);
+    }
+  }
+  float inv = 1.f;
+  if (norm_w) {
+    float sum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sum += x[i] * x[i] + y[i] * y[i];
+#pragma unroll
+    for (int offset = G / 2; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, EI_WAVE);
+    inv = rsqrtf(sum / static_cast<float>(D) + eps);
+  }
+  if (!active || !stored) return;
+  float ox[4], oy[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float a = x[i], b = y[i];
+    if (norm_w) {
+      a = (a * inv) * wx[i];
+      b = (b * inv) * wy[i];
+    }
+    if (rotate) {
+      const float ra = a * cs[i] - b * sn[i];
+      const float rb = a * sn[i] + b * cs[i];
+      a = ra;
+      b = rb;
+    }
+    ox[i] = a;
+    oy[i] = b;
+  }
+  Vec4<TO>::store(dst + i0, ox);
+  Vec4<TO>::store(dst + i0 + half, oy);
+}
+
 }  // namespace
 
 // qkv: [nsplit][N, (nq + 2 nkv) * D] of in_dtype.  q_out: [N, nq * D] of out_dtype.
@@ -128,11 +233,49 @@ extern "C" int ei_qk_norm_rope_store(
   EI_REQUIRE(nsplit >= 1, "qk_norm_rope_store: nsplit must be at least 1");
   (void)max_pos;
   const int heads = nq + 2 * nkv;
-  const long long waves = static_cast<long long>(N) * heads;
   const int threads = 256;
+  const size_t ss = static_cast<size_t>(split_stride);
+  // vector kernel: 4 pairs a lane, G = lanes a head (the power of two at or above D/8)
+  const bool aligned = (reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
+                        reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(v_pages) |
+                        reinterpret_cast<uintptr_t>(q_norm_w) | reinterpret_cast<uintptr_t>(k_norm_w) |
+                        reinterpret_cast<uintptr_t>(rope_table)) % 16 == 0;
+  if (D % 8 == 0 && ss % 4 == 0 && aligned) {
+    int G = 1;
+    while (G * 8 < D) G *= 2;
+    const long long items = static_cast<long long>(N) * heads;
+    const long long blocks = (items * G + threads - 1) / threads;
+    EI_REQUIRE(blocks < (1ll << 31), "qk_norm_rope_store: too many rows");
+#define EI_ROPE_VEC(TI, TO, GG)                                                                   \
+  qk_norm_rope_store_vec_kernel<TI, TO, GG><<<static_cast<unsigned>(blocks), threads, 0, stream>>>( \
+      static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, rope_table, row_pos,      \
+      row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),       \
+      static_cast<TO*>(v_pages), N, nq, nkv, D, write_cache)
+#define EI_ROPE_VEC_G(TI, TO)                                                                     \
+  do {                                                                                            \
+    if (G <= 2) EI_ROPE_VEC(TI, TO, 2);                                                           \
+    else if (G == 4) EI_ROPE_VEC(TI, TO, 4);                                                      \
+    else if (G == 8) EI_ROPE_VEC(TI, TO, 8);                                                      \
+    else if (G == 16) EI_ROPE_VEC(TI, TO, 16);                                                    \
+    else if (G == 32) EI_ROPE_VEC(TI, TO, 32);                                                    \
+    else EI_ROPE_VEC(TI, TO, 64);                                                                 \
+  } while (0)
+    if (G <= 2) G = 2;
+    if (in_dtype == EI_F32 && out_dtype == EI_F32)
+      EI_ROPE_VEC_G(float, float);
+    else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
+      EI_ROPE_VEC_G(float, bf16_t);
+    else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
+      EI_ROPE_VEC_G(bf16_t, bf16_t);
+    else
+      EI_REQUIRE(false, "qk_norm_rope_store: unsupported dtype combination");
+#undef EI_ROPE_VEC_G
+#undef EI_ROPE_VEC
+    EI_LAUNCH_CHECK();
+  }
+  const long long waves = static_cast<long long>(N) * heads;
   const long long blocks = (waves * EI_WAVE + threads - 1) / threads;
   EI_REQUIRE(blocks < (1ll << 31), "qk_norm_rope_store: too many rows");
-  const size_t ss = static_cast<size_t>(split_stride);
 #define EI_ROPE_LAUNCH(TI, TO)                                                                   \
   qk_norm_rope_store_kernel<TI, TO><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(      \
       static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, rope_table, row_pos,     \

@@ -62,29 +62,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
 
 // The same for widths that are a multiple of 4: 16-byte accesses, the row kept in
 // registers, up to 1024 threads a row so that few rows still have many loads in flight.
-template <typename T> struct Vec4;
-template <> struct Vec4<float> {
-  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
-    const float4 x = *reinterpret_cast<const float4*>(p);
-    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
-  }
-  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
-    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-  }
-};
-template <> struct Vec4<bf16_t> {
-  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[4]) {
-    const uint2 x = *reinterpret_cast<const uint2*>(p);
-    v[0] = __uint_as_float(x.x << 16); v[1] = __uint_as_float(x.x & 0xffff0000u);
-    v[2] = __uint_as_float(x.y << 16); v[3] = __uint_as_float(x.y & 0xffff0000u);
-  }
-  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[4]) {
-    uint2 x;
-    x.x = static_cast<uint32_t>(ei::f32_to_bf16(v[0])) | (static_cast<uint32_t>(ei::f32_to_bf16(v[1])) << 16);
-    x.y = static_cast<uint32_t>(ei::f32_to_bf16(v[2])) | (static_cast<uint32_t>(ei::f32_to_bf16(v[3])) << 16);
-    *reinterpret_cast<uint2*>(p) = x;
-  }
-};
+using ei::Vec4;
 
 template <typename TD, typename TO, bool HAS_DELTA, int CHUNKS>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
@@ -171,6 +149,16 @@ __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t
   }
 }
 
+// x / (1 + e^-x).  For a float32 result the library's exponential and a true division;
+// for a bfloat16 result (8 bits of mantissa) the hardware's exp2 and reciprocal, both good
+// to about one unit in the 23rd bit, which the rounding to bfloat16 swallows.
+template <typename TO> __device__ __forceinline__ float silu(float x);
+template <> __device__ __forceinline__ float silu<float>(float x) { return x / (1.0f + expf(-x)); }
+template <> __device__ __forceinline__ float silu<bf16_t>(float x) {
+  const float e = __builtin_amdgcn_exp2f(fmaxf(x, -80.f) * -1.44269504088896341f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
 // The same for I a multiple of 8: a thread takes 8 neighbouring columns of one row with
 // 16-byte (bfloat16) or 2 x 16-byte (float32) accesses.
 template <typename TI, typename TO>
@@ -212,8 +200,8 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
     float y0[4], y1[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      y0[i] = gate[i] / (1.0f + expf(-gate[i])) * up[i];
-      y1[i] = gate[i + 4] / (1.0f + expf(-gate[i + 4])) * up[i + 4];
+      y0[i] = silu<TO>(gate[i]) * up[i];
+      y1[i] = silu<TO>(gate[i + 4]) * up[i + 4];
     }
     TO* dst = out + row * I + col;
     Vec4<TO>::store(dst, y0);
@@ -268,8 +256,11 @@ static void launch_add_rmsnorm(float* residual, const void* delta, int nsplit, s
                                int N, int H, int write_residual, hipStream_t stream) {
   if (H % 4 == 0 && (!delta || split_stride % 4 == 0)) {
     const int quads = H / 4;
+    // few rows: up to 1024 threads a row, so that many loads are in flight; many rows: 256
+    // threads a row, so that several rows share a compute unit and overlap their phases
+    const int most = N >= 512 && quads <= 4 * 256 ? 256 : 1024;
     int threads = (quads + EI_WAVE - 1) / EI_WAVE * EI_WAVE;
-    if (threads > 1024) threads = 1024;
+    if (threads > most) threads = most;
     const int chunks = (quads + threads - 1) / threads;      // 1..4 for H <= 16384
 #define EI_NORM_VEC(C)                                                                         \
   do {                                                                                         \

@@ -161,9 +161,14 @@ class PagedCache:
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("form", ["slices", "stored"])
 @pytest.mark.parametrize("nq,nkv,D,use_norm,use_rope", [(6, 3, 48, True, True), (4, 4, 16, False, True),
-                                                        (8, 1, 256, True, False)])
-def test_qk_norm_rope_store(lib, dtype, nq, nkv, D, use_norm, use_rope):
+                                                        (8, 1, 256, True, False), (5, 1, 128, True, True),
+                                                        (3, 1, 20, True, True), (2, 2, 8, True, True)])
+def test_qk_norm_rope_store(lib, dtype, form, nq, nkv, D, use_norm, use_rope):
+    """Input as float32 partial sums (two slices, the decode form) or as one tensor of the
+    storage type (the prefill form); head sizes that take the vector kernel (multiples of
+    8, with idle lanes at 48) and one that takes the scalar kernel (20)."""
     theta, eps = 1e6, 1e-5
     lengths_before = [70, 0, 130]
     counts = [3, 5, 1]
@@ -172,6 +177,8 @@ def test_qk_norm_rope_store(lib, dtype, nq, nkv, D, use_norm, use_rope):
     sentinel_k, sentinel_v = cache.k.clone(), cache.v.clone()
     width = (nq + 2 * nkv) * D
     qkv = torch.randn(2, N, width, device=DEV)
+    if form == "stored":
+        qkv = qkv[0].to(dtype).unsqueeze(0)
     row_pos, row_seq = [], []
     for b, (start, count) in enumerate(zip(lengths_before, counts)):
         row_pos += list(range(start, start + count))
@@ -183,8 +190,8 @@ def test_qk_norm_rope_store(lib, dtype, nq, nkv, D, use_norm, use_rope):
     kn = (1 + 0.1 * torch.randn(D, device=DEV)) if use_norm else None
     table = rope_table(D, theta, 256) if use_rope else None
     q_out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=dtype)
-    lib.qk_norm_rope_store(qkv, qn, kn, eps, table, pos, seq, cache.table_dev, q_out, cache.k,
-                           cache.v, nq, nkv, D)
+    lib.qk_norm_rope_store(qkv if form == "slices" else qkv[0], qn, kn, eps, table, pos, seq,
+                           cache.table_dev, q_out, cache.k, cache.v, nq, nkv, D)
     total = qkv.double().cpu().sum(0)
     q = total[:, :nq * D].reshape(N, nq, D)
     k = total[:, nq * D:(nq + nkv) * D].reshape(N, nkv, D)
