@@ -65,7 +65,8 @@ _SIGNATURES = {
                                        c_void_p],
     },
     "sampling": {
-        "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
+        "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
+        "ei_argmax_partial_size": [c_int, c_int],
         "ei_sample": [c_void_p, c_int, c_int, c_float, c_float, c_int, c_ulonglong, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p],
     },
@@ -360,7 +361,13 @@ def gemm_f32(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     _check(lib, status, "gemm_f32")
 
 
-def argmax(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None) -> None:
+def argmax_partial_size(rows: int, vocab: int) -> int:
+    """float32 elements of scratch with which `argmax` searches a wide vocabulary with many
+    blocks a row (0: one block a row is used anyway)."""
+    return 2 * library("sampling").ei_argmax_partial_size(rows, vocab)
+
+
+def argmax(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None, partial=None) -> None:
     lib = library("sampling")
     rows, vocab = logits.shape
     if tokens.numel() < rows:
@@ -368,7 +375,9 @@ def argmax(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None) -> No
     status = lib.ei_argmax(_gpu(logits, "logits", torch.float32), rows, vocab,
                            _gpu(tokens, "tokens", torch.int32),
                            None if probabilities is None
-                           else _gpu(probabilities, "probabilities", torch.float32), _stream())
+                           else _gpu(probabilities, "probabilities", torch.float32),
+                           None if partial is None else _gpu(partial, "partial", torch.float32),
+                           0 if partial is None else partial.numel() // 2, _stream())
     _check(lib, status, "argmax")
 
 

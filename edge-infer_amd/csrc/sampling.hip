@@ -84,6 +84,74 @@ argmax_kernel(const float* __restrict__ logits, int V, int32_t* __restrict__ tok
   }
 }
 
+// Wide vocabularies, two steps: every block finds the best of one chunk of a row, then one
+// wave a row picks the best chunk.  The same order (larger value, then lower index) as above.
+constexpr int kArgmaxThreads = 256;
+constexpr int kArgmaxChunk = 4096;
+
+__device__ __forceinline__ void keep_better(float& value, int& index, float other_value,
+                                            int other_index) {
+  if (other_value > value || (other_value == value && other_index < index)) {
+    value = other_value;
+    index = other_index;
+  }
+}
+
+__global__ void __launch_bounds__(kArgmaxThreads)
+argmax_chunks_kernel(const float* __restrict__ logits, int V, float2* __restrict__ partial) {
+  __shared__ float best_value[kArgmaxThreads / EI_WAVE];
+  __shared__ int best_index[kArgmaxThreads / EI_WAVE];
+  const float* row = logits + static_cast<size_t>(blockIdx.y) * V;
+  const int begin = blockIdx.x * kArgmaxChunk;
+  const int end = min(V, begin + kArgmaxChunk);
+  float value = -INFINITY;
+  int index = 0x7fffffff;
+  constexpr int kPerThread = kArgmaxChunk / kArgmaxThreads;
+  float z[kPerThread];
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {          // all loads first
+    const int i = begin + threadIdx.x + j * kArgmaxThreads;
+    z[j] = i < end ? row[i] : -INFINITY;
+  }
+#pragma unroll
+  for (int j = 0; j < kPerThread; ++j) {
+    const int i = begin + threadIdx.x + j * kArgmaxThreads;
+    if (i < end) keep_better(value, index, scaled_logit(z[j], 1.f, false), i);
+  }
+#pragma unroll
+  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1)
+    keep_better(value, index, __shfl_xor(value, offset, EI_WAVE), __shfl_xor(index, offset, EI_WAVE));
+  const int wave = threadIdx.x / EI_WAVE, lane = threadIdx.x % EI_WAVE;
+  if (lane == 0) {
+    best_value[wave] = value;
+    best_index[wave] = index;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int w = 1; w < kArgmaxThreads / EI_WAVE; ++w)
+      keep_better(value, index, best_value[w], best_index[w]);
+    partial[static_cast<size_t>(blockIdx.y) * gridDim.x + blockIdx.x] =
+        make_float2(value, __int_as_float(index));
+  }
+}
+
+__global__ void __launch_bounds__(EI_WAVE)
+argmax_merge_kernel(const float2* __restrict__ partial, int chunks, int32_t* __restrict__ tokens,
+                    float* __restrict__ probabilities) {
+  const float2* mine = partial + static_cast<size_t>(blockIdx.x) * chunks;
+  float value = -INFINITY;
+  int index = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += EI_WAVE)
+    keep_better(value, index, mine[c].x, __float_as_int(mine[c].y));
+#pragma unroll
+  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1)
+    keep_better(value, index, __shfl_xor(value, offset, EI_WAVE), __shfl_xor(index, offset, EI_WAVE));
+  if (threadIdx.x == 0) {
+    tokens[blockIdx.x] = index == 0x7fffffff ? 0 : index;
+    if (probabilities) probabilities[blockIdx.x] = 1.f;
+  }
+}
+
 __global__ void __launch_bounds__(kThreads)
 sample_kernel(const float* __restrict__ logits, int V, float temperature, float top_p, int top_k,
               uint64_t seed, const int32_t* __restrict__ streams,
@@ -249,10 +317,30 @@ sample_kernel(const float* __restrict__ logits, int V, float temperature, float 
 
 }  // namespace
 
+// Elements of `partial` (float2) that ei_argmax wants for these sizes; 0: it needs none.
+extern "C" int ei_argmax_partial_size(int rows, int V) {
+  if (rows < 1 || V <= 2 * kArgmaxChunk) return 0;
+  const long long size = static_cast<long long>(rows) * ((V + kArgmaxChunk - 1) / kArgmaxChunk);
+  return size < (1ll << 30) ? static_cast<int>(size) : 0;
+}
+
+// `partial` (float2 [rows, chunks], or null) lets a wide vocabulary be searched by many
+// blocks a row; without it one block takes a row.  The result is the same either way.
 extern "C" int ei_argmax(const float* logits, int rows, int V, int32_t* tokens,
-                         float* probabilities, hipStream_t stream) {
+                         float* probabilities, void* partial, long long partial_size,
+                         hipStream_t stream) {
   EI_REQUIRE(rows > 0 && V > 0, "argmax: sizes must be positive");
   EI_REQUIRE(logits && tokens, "argmax: null pointer");
+  const int want = ei_argmax_partial_size(rows, V);
+  if (partial && want > 0) {
+    EI_REQUIRE(partial_size >= want, "argmax: the partial buffer is too small");
+    const int chunks = (V + kArgmaxChunk - 1) / kArgmaxChunk;
+    argmax_chunks_kernel<<<dim3(chunks, rows), kArgmaxThreads, 0, stream>>>(
+        logits, V, static_cast<float2*>(partial));
+    argmax_merge_kernel<<<rows, EI_WAVE, 0, stream>>>(static_cast<const float2*>(partial), chunks,
+                                                      tokens, probabilities);
+    EI_LAUNCH_CHECK();
+  }
   argmax_kernel<<<rows, kThreads, 0, stream>>>(logits, V, tokens, probabilities);
   EI_LAUNCH_CHECK();
 }

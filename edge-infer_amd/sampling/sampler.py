@@ -19,6 +19,7 @@ class Sampler:
         self._tokens = torch.empty(1024, dtype=torch.int32, device=self.device)
         self._probabilities = torch.empty(1024, dtype=torch.float32, device=self.device)
         self._meta = torch.empty(2048, dtype=torch.int32, device=self.device)
+        self._partial = None          # scratch of the greedy search over a wide vocabulary
         self._last_rows = 0
 
     def _reserve(self, rows: int) -> None:
@@ -36,7 +37,10 @@ class Sampler:
         tokens = self._tokens[:rows]
         probabilities = self._probabilities[:rows]
         if params.is_greedy(vocab):
-            lib.argmax(logits, tokens, probabilities)
+            need = lib.argmax_partial_size(rows, vocab)
+            if need and (self._partial is None or self._partial.numel() < need):
+                self._partial = torch.empty(need, dtype=torch.float32, device=self.device)
+            lib.argmax(logits, tokens, probabilities, self._partial if need else None)
         else:
             if len(streams) != rows or len(counters) != rows:
                 raise ValueError("one stream number and one counter per row are needed")

@@ -446,6 +446,27 @@ def test_argmax_ties_and_nan(lib):
     tokens = torch.empty(3, dtype=torch.int32, device=DEV)
     lib.argmax(big, tokens)
     assert tokens.tolist() == [int(big[0].argmax()), 77, int(big[2].argmax())]
+    # the same through many blocks a row: ties across chunks, NaN, a width that ends inside
+    # a chunk, an all -inf row
+    for vocab in (151936, 8193, 12288):
+        big = torch.randn(5, vocab, device=DEV)
+        big[1, vocab - 1] = 9.0
+        big[1, 4097] = 9.0
+        big[2, 5000] = float("nan")
+        big[3] = float("-inf")
+        big[4, vocab - 1] = 11.0
+        need = lib.argmax_partial_size(5, vocab)
+        assert need > 0
+        partial = torch.full((need,), float("nan"), device=DEV)
+        tokens = torch.full((5,), -1, dtype=torch.int32, device=DEV)
+        prob = torch.zeros(5, device=DEV)
+        lib.argmax(big, tokens, prob, partial)
+        finite = torch.nan_to_num(big[2], nan=float("-inf"))
+        assert tokens.tolist() == [int(big[0].argmax()), 4097, int(finite.argmax()), 0, vocab - 1]
+        assert prob.tolist() == [1.0] * 5
+        with pytest.raises(lib.KernelError, match="too small"):
+            lib.argmax(big, tokens, prob, partial[:need - 2])
+    assert lib.argmax_partial_size(4, 8192) == 0
 
 
 def test_sample_reference_distribution(lib):
