@@ -1,21 +1,22 @@
 // Weight-streaming matrix product for few rows (decode): out[s][m][n] = partial sums of
 // X[m, :] . W[n, :] over the s-th slice of K, for M <= 64 rows of X.
 //
-// W is a bfloat16 checkpoint matrix in its stored [N, K] layout and is read exactly once,
-// straight from global memory into MFMA operand registers: with v_mfma_f32_16x16x32_bf16 a
-// lane supplies 8 consecutive k of one row, and because a dot product does not care in
-// which order k is visited, lane (row r, quarter c) takes the contiguous run
-// k0 + c*KT/4 .. + KT/4 of its row and feeds it to successive MFMAs, eight elements at a
-// time.  X (tiny) is staged through LDS once per workgroup and K-tile and read with the same
-// k mapping; the next tiles of W and X are already on their way while a tile is multiplied.  A workgroup is 4 waves, each owning 16 rows of W; K may be split over
-// blockIdx.y, in which case every slice writes float32 partial sums [slice, M, N] that the
-// consuming kernel adds in slice order while it reads them (deterministic, no atomics, and
-// no device-wide fence: the kernel boundary orders the writes before the reads).
+// W is a bfloat16 checkpoint matrix [N, K] and is read exactly once, straight from global
+// memory into MFMA operand registers (v_mfma_f32_16x16x32_bf16: lane (row r, quarter c) holds
+// 8 consecutive k of row r).  It is read either in its stored layout or, faster, from a copy
+// packed at load time into whole MFMA tiles (see ei_gemm_bf16_skinny_packed).  X (tiny) is
+// staged through LDS one K-tile at a time.  A workgroup is 4, 6 or 8 waves, each owning 16
+// rows of W; K may be split over blockIdx.y, in which case every slice writes float32 partial
+// sums [slice, M, N] that the consuming kernel adds in slice order while it reads them
+// (deterministic, no atomics, and no device-wide fence: the kernel boundary orders the
+// writes before the reads).  The host picks the waves and slices per shape.
 //
 // Accumulation is float32 throughout, as in the reference's cublasGemmEx call
 // (operators/src/cuda/execution.cu:319-323); the sums stay float32 and the consumer rounds
 // once when it stores in the storage type.
 #include "common.cuh"
+
+#include <type_traits>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -23,9 +24,6 @@ typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * EI_WAVE;
-constexpr int kRowsPerBlock = kWaves * 16;
 constexpr int kPackedTile = 16 * 32;      // elements of one packed tile: 16 rows x 32 k, 1 KB
 
 // Address of the 16-byte piece that lane `lane` takes of the packed tile (kt, strip).
@@ -34,25 +32,35 @@ __device__ __forceinline__ const bf16_t* packed_piece(const bf16_t* Wp, int n_st
   return Wp + (static_cast<size_t>(kt) * n_strips + strip) * kPackedTile + lane * 8;
 }
 
-template <int MB, int KT, bool PACKED>
-__global__ void __launch_bounds__(kThreads)
+// Up to 64 rows of X, any K range.  A workgroup is WAVES waves, each owning 16 rows of W; X
+// travels through LDS one K-tile (256) at a time, two tiles of it alternate so that a tile
+// costs one barrier.  W has two register sets that are refilled piece by piece: as soon as
+// the products of one 32-wide step have read their piece, the same piece of the tile after
+// next is requested, so two tiles of W per wave are always on their way.  The loads of the
+// steady loop are unconditional (clamped addresses, zeros selected afterwards), so the number
+// outstanding is the same on every path and each wait leaves the younger loads in flight.
+// Few K slices: for many rows the float32 partial sums (rows x N x 4 bytes a slice, written
+// in 64-byte pieces and read again by the consumer) cost more than the weights they save.
+template <int MB, int WAVES, bool PACKED>
+__global__ void __launch_bounds__(WAVES * EI_WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
                    float* __restrict__ out, int M, int N, int K, int k_per_split) {
-  constexpr int JN = KT / 32;             // MFMA steps per K-tile
+  constexpr int KT = 256, JN = KT / 32;   // MFMA steps per K-tile
+  constexpr int THREADS = WAVES * EI_WAVE;
   constexpr int ROWS_X = MB * 16;
   constexpr int XS = KT + 8;              // LDS row stride in elements (16 bytes of padding)
   constexpr int CHUNKS = ROWS_X * (KT / 8);
-  constexpr int XLOADS = CHUNKS / kThreads;
-  static_assert(CHUNKS % kThreads == 0, "X tile must divide among the threads");
-  __shared__ __attribute__((aligned(16))) bf16_t xs[ROWS_X * XS];
+  constexpr int XLOADS = (CHUNKS + THREADS - 1) / THREADS;
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS_X * XS];
 
   const int t = threadIdx.x;
   const int wave = t / EI_WAVE, lane = t % EI_WAVE;
   const int r16 = lane & 15, c = lane >> 4;
-  const int n_tile = blockIdx.x * kRowsPerBlock + wave * 16;
+  const int n_tile = (blockIdx.x * WAVES + wave) * 16;
   const int k_begin = blockIdx.y * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
   const int n_iter = (k_end - k_begin + KT - 1) / KT;
+  if (n_iter <= 0) return;
 
   int w_row = n_tile + r16;
   if (w_row >= N) w_row = N - 1;          // rows past the end repeat the last one; never stored
@@ -66,82 +74,116 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 w_a[JN], w_b[JN];
+  bf16x8 w[2][JN];
   u32x4 x_regs[XLOADS];
   const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
 
-  auto load_w = [&](bf16x8* dst, int kb) {
-#pragma unroll
-    for (int j = 0; j < JN; ++j) {
-      if (PACKED) {
-        // the packed copy holds whole K-tiles (zeros past K): no test, so that the loads
-        // form one straight run whose arrival the compiler can count
-        dst[j] = __builtin_nontemporal_load(
-            reinterpret_cast<const bf16x8*>(w_ptr + (kb / 32 + j) * tile_stride));
-        continue;
-      }
-      const int k = kb + j * 32 + c * 8;
-      if (k < k_end) {
-        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
-      } else {
-        dst[j] = __builtin_bit_cast(bf16x8, zero4);
-      }
+  auto load_w_piece = [&](int set, int tile, int j) {
+    const int kb = k_begin + tile * KT;
+    if (PACKED) {
+      // the packed copy holds whole K-tiles (zeros past K): no test
+      w[set][j] = __builtin_nontemporal_load(
+          reinterpret_cast<const bf16x8*>(w_ptr + (kb / 32 + j) * tile_stride));
+    } else {
+      // clamped to the last piece of the slice; the matching piece of X is zero there
+      const int k = min(kb + j * 32 + c * 8, k_end - 8);
+      w[set][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + k - c * 8));
     }
   };
-  auto load_x = [&](int kb) {
+  auto load_x = [&](int tile) {
+    const int kb = k_begin + tile * KT;
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
-      const int q = t + i * kThreads;
-      const int row = q / (KT / 8), ch = q % (KT / 8);
-      const int k = kb + ch * 8;
-      x_regs[i] = (row < M && k < k_end)
-                      ? *reinterpret_cast<const u32x4*>(X + static_cast<size_t>(row) * K + k)
-                      : zero4;
+      const int q = t + i * THREADS;
+      const int row = q / (KT / 8), k = kb + (q % (KT / 8)) * 8;
+      const bool valid = row < M && k < k_end;
+      x_regs[i] = *reinterpret_cast<const u32x4*>(
+          X + static_cast<size_t>(valid ? row : 0) * K + (valid ? k : k_begin));
     }
   };
-  auto store_x = [&]() {
+  auto store_x = [&](int buf, int tile) {
+    const int kb = k_begin + tile * KT;
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
-      const int q = t + i * kThreads;
+      const int q = t + i * THREADS;
       const int row = q / (KT / 8), ch = q % (KT / 8);
-      *reinterpret_cast<u32x4*>(&xs[row * XS + ch * 8]) = x_regs[i];
+      const bool valid = row < M && kb + ch * 8 < k_end;
+      if (CHUNKS % THREADS == 0 || q < CHUNKS)
+        *reinterpret_cast<u32x4*>(&xs[buf][row * XS + ch * 8]) = valid ? x_regs[i] : zero4;
     }
   };
-  auto compute = [&](const bf16x8* w) {
+  // products of a tile whose W is in register set `set` and whose X is in LDS buffer `set`
+  // (even tiles 0, odd tiles 1); refill >= 0: request every piece of that tile into the set
+  // that is being used up.  `set` is a constant at every call, so that the sets stay registers.
+  auto compute = [&](auto set_tag, auto refill_tag, int refill) {
+    constexpr int set = decltype(set_tag)::value;
+    constexpr bool do_refill = decltype(refill_tag)::value;
+    const bf16_t* x_base = &xs[set][r16 * XS + c * 8];
+    bf16x8 xf[2][MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+      xf[0][mb] = *reinterpret_cast<const bf16x8*>(x_base + mb * 16 * XS);
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
+      if (j + 1 < JN) {
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        const bf16x8 xv = *reinterpret_cast<const bf16x8*>(
-            &xs[(mb * 16 + r16) * XS + j * 32 + c * 8]);
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j], xv, acc[mb], 0, 0, 0);
+        for (int mb = 0; mb < MB; ++mb)
+          xf[(j + 1) & 1][mb] =
+              *reinterpret_cast<const bf16x8*>(x_base + mb * 16 * XS + (j + 1) * 32);
       }
+      // keep this order (reads of the next step, products, refill): left alone the
+      // scheduler pairs every read with its use and gathers the refills at the end
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[set][j], xf[j & 1][mb], acc[mb], 0, 0, 0);
+      if (do_refill) load_w_piece(set, refill, j);
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // Two register sets for W alternate, so that a tile is never copied (a copy would wait
-  // for its loads at once); the next tiles of W and X travel while this one is multiplied.
-  if (n_iter > 0) {
-    load_w(w_a, k_begin);
-    load_x(k_begin);
-  }
-  for (int it = 0; it < n_iter; it += 2) {
-    __syncthreads();                      // the previous tile of X has been read by everyone
-    store_x();
+  using Set0 = std::integral_constant<int, 0>;
+  using Set1 = std::integral_constant<int, 1>;
+  using Refill = std::true_type;
+  using Last = std::false_type;
+
+  load_x(0);
+#pragma unroll
+  for (int j = 0; j < JN; ++j) load_w_piece(0, 0, j);
+  if (n_iter == 1) {
+    store_x(0, 0);
     __syncthreads();
-    if (it + 1 < n_iter) {
-      load_w(w_b, k_begin + (it + 1) * KT);
-      load_x(k_begin + (it + 1) * KT);
+    compute(Set0{}, Last{}, 0);
+  } else {
+#pragma unroll
+    for (int j = 0; j < JN; ++j) load_w_piece(1, 1, j);
+    store_x(0, 0);
+    load_x(1);
+    __syncthreads();
+    int i = 0;                            // even: tile i is in set 0
+    for (; i + 3 < n_iter; i += 2) {      // tiles i + 2 and i + 3 exist
+      compute(Set0{}, Refill{}, i + 2);
+      store_x(1, i + 1);
+      load_x(i + 2);
+      __syncthreads();
+      compute(Set1{}, Refill{}, i + 3);
+      store_x(0, i + 2);
+      load_x(i + 3);
+      __syncthreads();
     }
-    compute(w_a);
-    if (it + 1 < n_iter) {
+    if (i + 2 < n_iter) {                 // three tiles remain
+      compute(Set0{}, Refill{}, i + 2);
+      store_x(1, i + 1);
+      load_x(i + 2);
       __syncthreads();
-      store_x();
+      compute(Set1{}, Last{}, 0);
+      store_x(0, i + 2);
       __syncthreads();
-      if (it + 2 < n_iter) {
-        load_w(w_a, k_begin + (it + 2) * KT);
-        load_x(k_begin + (it + 2) * KT);
-      }
-      compute(w_b);
+      compute(Set0{}, Last{}, 0);
+    } else {                              // two
+      compute(Set0{}, Last{}, 0);
+      store_x(1, i + 1);
+      __syncthreads();
+      compute(Set1{}, Last{}, 0);
     }
   }
 
@@ -163,173 +205,80 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   }
 }
 
-// Up to 16 rows of X and a K range of at most kPreloadK: the whole X slice is put into LDS
-// once, after which the four waves stream their rows of W without meeting again.
-constexpr int kPreloadK = 1024;
+constexpr int kTile = 256;                // K-tile of the kernel
+constexpr int kComputeUnits = 256;        // MI355X
 
-template <bool PACKED>
-__global__ void __launch_bounds__(kThreads)
-skinny_gemm_preload_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
-                           float* __restrict__ out, int M, int N, int K, int k_per_split,
-                           int row_tiles) {
-  constexpr int KT = 256, JN = KT / 32;
-  constexpr int XS = kPreloadK + 8;
-  __shared__ __attribute__((aligned(16))) bf16_t xs[16 * XS];
-
-  const int t = threadIdx.x;
-  const int wave = t / EI_WAVE, lane = t % EI_WAVE;
-  const int r16 = lane & 15, c = lane >> 4;
-  const int k_begin = blockIdx.y * k_per_split;
-  const int k_end = min(K, k_begin + k_per_split);
-  const int k_len = k_end - k_begin;                 // a multiple of 8, at most kPreloadK
-  const int n_iter = (k_len + KT - 1) / KT;
-
-  // X slice -> LDS: 16 rows (zeros past M and past the slice), 16-byte chunks, at most 8
-  // per thread.  Every load is issued (from a clamped address) before the first is used.
-  const u32x4 zero4 = u32x4{0u, 0u, 0u, 0u};
-  const int chunks_per_row = n_iter * (KT / 8);
-  constexpr int XCH = 16 * (kPreloadK / 8) / kThreads;
-  u32x4 xv[XCH];
-#pragma unroll
-  for (int i = 0; i < XCH; ++i) {
-    const int q = t + i * kThreads;
-    const int row = q / chunks_per_row, k = (q % chunks_per_row) * 8;
-    const bool valid = row < M && k < k_len;
-    const u32x4 v = *reinterpret_cast<const u32x4*>(
-        X + static_cast<size_t>(valid ? row : 0) * K + k_begin + (valid ? k : 0));
-    xv[i] = valid ? v : zero4;
+// Waves per block (4, 6 or 8) and what the busiest compute unit then has to do, in strips:
+// `strips * splits` strip-slices are dealt out in blocks of `waves` strips.  Up to two blocks
+// per unit all run at once, so the unit with the most blocks sets the time; many more blocks
+// than that even out.  Every block also costs a start (about 3 strip-tiles).  Ties go to the
+// larger block, which shares a tile of X among more waves.
+int tile_kernel_waves(int n_strips, int splits, double tiles_per_slice, double* cost_out) {
+  int best = 8;
+  double best_cost = 1e30;
+  for (int waves = 8; waves >= 4; waves -= 2) {
+    const double blocks = static_cast<double>((n_strips + waves - 1) / waves) * splits;
+    const double per_unit = blocks <= 2 * kComputeUnits
+                                ? static_cast<double>((static_cast<long long>(blocks) + kComputeUnits - 1) / kComputeUnits)
+                                : blocks / kComputeUnits + 0.25;
+    const double cost = per_unit * (waves * tiles_per_slice + 3.0);
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = waves;
+    }
   }
-  auto store_x = [&]() {                               // after the first loads of W are issued
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) {
-      const int q = t + i * kThreads;
-      const int row = q / chunks_per_row, k = (q % chunks_per_row) * 8;
-      if (row < 16) *reinterpret_cast<u32x4*>(&xs[row * XS + k]) = xv[i];
-    }
-  };
-  const bf16_t* x_ptr = &xs[r16 * XS + c * 8];
-
-  // The block owns `row_tiles` consecutive groups of 64 rows of W (16 per wave); the walk
-  // over (group, K-tile) is one flat pipeline with two tiles of W in flight per wave.
-  const int first_group = blockIdx.x * row_tiles;
-  const int total = row_tiles * n_iter;
-  const int n_strips = (N + 15) / 16;
-  const size_t tile_stride = static_cast<size_t>(n_strips) * kPackedTile;
-  auto w_pointer = [&](int group) {
-    if (PACKED) {
-      const int strip = min((first_group + group) * kWaves + wave, n_strips - 1);
-      return packed_piece(W, n_strips, k_begin / 32, strip, lane);
-    }
-    int row = (first_group + group) * kRowsPerBlock + wave * 16 + r16;
-    if (row >= N) row = N - 1;                        // repeats the last row; never stored
-    return W + static_cast<size_t>(row) * K + k_begin + c * 8;
-  };
-  bf16x8 w_a[JN], w_b[JN];
-  auto load_w = [&](bf16x8* dst, int step) {          // step = group * n_iter + tile
-    const bf16_t* w_ptr = w_pointer(step / n_iter);
-    const int kb = (step % n_iter) * KT;
-#pragma unroll
-    for (int j = 0; j < JN; ++j) {
-      if (PACKED) {
-        dst[j] = __builtin_nontemporal_load(
-            reinterpret_cast<const bf16x8*>(w_ptr + (kb / 32 + j) * tile_stride));
-        continue;
-      }
-      if (kb + j * 32 + c * 8 < k_len) {
-        dst[j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + kb + j * 32));
-      } else {
-        dst[j] = __builtin_bit_cast(bf16x8, zero4);
-      }
-    }
-  };
-  f32x4 acc0 = f32x4{0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
-  float* dst = out + static_cast<size_t>(blockIdx.y) * M * N;
-  auto compute = [&](const bf16x8* w, int step) {
-    const int kb = (step % n_iter) * KT;
-#pragma unroll
-    for (int j = 0; j < JN; j += 2) {
-      const bf16x8 x0 = *reinterpret_cast<const bf16x8*>(x_ptr + kb + j * 32);
-      const bf16x8 x1 = *reinterpret_cast<const bf16x8*>(x_ptr + kb + (j + 1) * 32);
-      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j], x0, acc0, 0, 0, 0);
-      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[j + 1], x1, acc1, 0, 0, 0);
-    }
-    if (step % n_iter == n_iter - 1) {                // a group of rows is complete
-      const f32x4 acc = acc0 + acc1;
-      acc0 = acc1 = f32x4{0.f, 0.f, 0.f, 0.f};
-      const int n0 = (first_group + step / n_iter) * kRowsPerBlock + wave * 16 + 4 * c;
-      if (r16 < M) {
-        float* p = dst + static_cast<size_t>(r16) * N + n0;
-        if (n0 + 3 < N && (N & 3) == 0) {
-          *reinterpret_cast<f32x4*>(p) = acc;
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (n0 + r < N) p[r] = acc[r];
-        }
-      }
-    }
-  };
-  // The loads of the steady loop are unconditional, so that on every path into a product
-  // the same number of loads is outstanding and the wait before it can let the younger
-  // tile stay in flight; the last two or three steps are peeled off.
-  if (total == 1) {
-    load_w(w_a, 0);
-    store_x();
-    __syncthreads();
-    compute(w_a, 0);
-    return;
-  }
-  load_w(w_a, 0);
-  load_w(w_b, 1);
-  store_x();
-  __syncthreads();
-  int step = 0;
-  for (; step + 3 < total; step += 2) {
-    compute(w_a, step);
-    load_w(w_a, step + 2);
-    compute(w_b, step + 1);
-    load_w(w_b, step + 3);
-  }
-  compute(w_a, step);
-  if (step + 2 < total) {
-    load_w(w_a, step + 2);
-    compute(w_b, step + 1);
-    compute(w_a, step + 2);
-  } else {
-    compute(w_b, step + 1);
-  }
+  if (cost_out) *cost_out = best_cost;
+  return best;
 }
 
-int tile_for(int MB) { (void)MB; return 256; }
+bool valid_slice_count(int k_tiles, int splits) {
+  if (splits < 1 || splits > k_tiles) return false;
+  const int per = (k_tiles + splits - 1) / splits;
+  return (k_tiles + per - 1) / per == splits;
+}
 
 }  // namespace
 
-// The number of K slices the kernel will use for these sizes (the caller sizes `out`).
-// More slices for fewer rows: the partial sums cost M * N * 8 bytes of traffic per slice.
-extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int target_blocks) {
+// The number of K slices the kernel will use for these sizes (the caller sizes `out`): the
+// count that leaves the busiest compute unit the least to do, where a slice's partial sums
+// (rows * N * 4 bytes, written in small pieces and read again by the consumer) are priced at
+// 2.5 times their size.  `max_splits` > 0 caps it.
+extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int max_splits) {
   if (M < 1 || N < 1 || K < 1) return 1;
-  const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int KT = tile_for(MB);
-  const int row_blocks = (N + kRowsPerBlock - 1) / kRowsPerBlock;
-  const int k_tiles = (K + KT - 1) / KT;
-  if (target_blocks <= 0) target_blocks = 512;
-  int splits = (target_blocks + row_blocks - 1) / row_blocks;
-  const int max_splits = MB == 1 ? 16 : (MB == 2 ? 8 : 4);
-  if (splits > max_splits) splits = max_splits;
-  if (MB == 1) {
-    // slices of at most kPreloadK let the kernel keep its X slice in LDS
-    const int need = (K + kPreloadK - 1) / kPreloadK;
-    if (splits < need && need <= 16) splits = need;
+  const int k_tiles = (K + kTile - 1) / kTile;
+  const int n_strips = (N + 15) / 16;
+  if (max_splits <= 0 || max_splits > 16) max_splits = 16;
+  int best = 1;
+  double best_cost = 1e30;
+  for (int splits = 1; splits <= max_splits && splits <= k_tiles; ++splits) {
+    if (!valid_slice_count(k_tiles, splits)) continue;
+    const double tiles = static_cast<double>((k_tiles + splits - 1) / splits);
+    double cost = 0.0;                                   // in strip-tiles (8 KB of W) per unit
+    tile_kernel_waves(n_strips, splits, tiles, &cost);
+    cost += 2.5 * splits * static_cast<double>(M) * N * 4.0 / kComputeUnits / 8192.0;
+    if (cost < best_cost - 1e-9) {
+      best_cost = cost;
+      best = splits;
+    }
   }
-  if (splits > k_tiles) splits = k_tiles;
-  if (splits < 1) splits = 1;
-  const int tiles_per_split = (k_tiles + splits - 1) / splits;
-  return (k_tiles + tiles_per_split - 1) / tiles_per_split;
+  return best;
 }
 
-// X: [M, K] bfloat16, W: [N, K] bfloat16, out: [splits, M, N] float32 (slice s holds the
-// sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 64.
 namespace {
+
+template <int MB, bool PACKED>
+void launch_tile_kernel(const bf16_t* w, const bf16_t* x, float* out, int M, int N, int K,
+                        int k_per_split, int splits, hipStream_t stream) {
+  const int n_strips = (N + 15) / 16;
+  const int waves = tile_kernel_waves(n_strips, splits, k_per_split / static_cast<double>(kTile), nullptr);
+  dim3 grid((n_strips + waves - 1) / waves, splits);
+  if (waves == 4)
+    skinny_gemm_kernel<MB, 4, PACKED><<<grid, 4 * EI_WAVE, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+  else if (waves == 6)
+    skinny_gemm_kernel<MB, 6, PACKED><<<grid, 6 * EI_WAVE, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+  else
+    skinny_gemm_kernel<MB, 8, PACKED><<<grid, 8 * EI_WAVE, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+}
 
 template <bool PACKED>
 int launch_skinny(const void* X, const void* W, float* out, int M, int N, int K, int splits,
@@ -342,33 +291,19 @@ int launch_skinny(const void* X, const void* W, float* out, int M, int N, int K,
                  (reinterpret_cast<uintptr_t>(out) & 15) == 0,
              "gemm_bf16_skinny: pointers must be 16-byte aligned");
   const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int KT = tile_for(MB);
-  const int k_tiles = (K + KT - 1) / KT;
+  const int k_tiles = (K + kTile - 1) / kTile;
   EI_REQUIRE(splits >= 1 && splits <= k_tiles, "gemm_bf16_skinny: bad slice count");
-  const int tiles_per_split = (k_tiles + splits - 1) / splits;
-  EI_REQUIRE((k_tiles + tiles_per_split - 1) / tiles_per_split == splits,
-             "gemm_bf16_skinny: slice count leaves an empty slice");
-  const int k_per_split = tiles_per_split * KT;
-  const int row_blocks = (N + kRowsPerBlock - 1) / kRowsPerBlock;
-  dim3 grid(row_blocks, splits);
+  EI_REQUIRE(valid_slice_count(k_tiles, splits), "gemm_bf16_skinny: slice count leaves an empty slice");
+  const int k_per_split = (k_tiles + splits - 1) / splits * kTile;
   const bf16_t* x = static_cast<const bf16_t*>(X);
   const bf16_t* w = static_cast<const bf16_t*>(W);
-  if (MB == 1 && k_per_split <= kPreloadK) {
-    // fat blocks for tall matrices: several groups of 64 rows share one staged X slice,
-    // as long as some 768 blocks remain
-    int row_tiles = static_cast<int>(static_cast<long long>(row_blocks) * splits / 768);
-    if (row_tiles < 1) row_tiles = 1;
-    if (row_tiles > 8) row_tiles = 8;
-    dim3 fat((row_blocks + row_tiles - 1) / row_tiles, splits);
-    skinny_gemm_preload_kernel<PACKED><<<fat, kThreads, 0, stream>>>(w, x, out, M, N, K,
-                                                                     k_per_split, row_tiles);
+  if (MB == 1) {
+    launch_tile_kernel<1, PACKED>(w, x, out, M, N, K, k_per_split, splits, stream);
+  } else if (MB == 2) {
+    launch_tile_kernel<2, PACKED>(w, x, out, M, N, K, k_per_split, splits, stream);
+  } else {
+    launch_tile_kernel<4, PACKED>(w, x, out, M, N, K, k_per_split, splits, stream);
   }
-  else if (MB == 1)
-    skinny_gemm_kernel<1, 256, PACKED><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
-  else if (MB == 2)
-    skinny_gemm_kernel<2, 256, PACKED><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
-  else
-    skinny_gemm_kernel<4, 256, PACKED><<<grid, kThreads, 0, stream>>>(w, x, out, M, N, K, k_per_split);
   EI_LAUNCH_CHECK();
 }
 

@@ -402,12 +402,12 @@ def has_skinny_gemm() -> bool:
     return "gemm_bf16" in build.available_libraries()
 
 
-_SKINNY_TARGET = int(os.environ.get("EDGE_INFER_SKINNY_BLOCKS", "0"))
+_SKINNY_MAX_SPLITS = int(os.environ.get("EDGE_INFER_SKINNY_MAX_SPLITS", "0"))   # 0: no cap
 
 
 def skinny_gemm_splits(rows: int, n: int, k: int) -> int:
     """K slices the weight-streaming product uses for [rows, k] x [n, k]^T."""
-    return library("gemm_bf16").ei_skinny_gemm_splits(rows, n, k, _SKINNY_TARGET)
+    return library("gemm_bf16").ei_skinny_gemm_splits(rows, n, k, _SKINNY_MAX_SPLITS)
 
 
 def skinny_gemm_ok(rows: int, k: int) -> bool:
