@@ -60,6 +60,16 @@ template <> struct Vec4<bf16_t> {
   }
 };
 
+// x / (1 + e^-x).  For a float32 result the library's exponential and a true division;
+// for a bfloat16 result (8 bits of mantissa) the hardware's exp2 and reciprocal, both good
+// to about one unit in the 23rd bit, which the rounding to bfloat16 swallows.
+template <typename TO> __device__ __forceinline__ float silu(float x);
+template <> __device__ __forceinline__ float silu<float>(float x) { return x / (1.0f + expf(-x)); }
+template <> __device__ __forceinline__ float silu<bf16_t>(float x) {
+  const float e = __builtin_amdgcn_exp2f(fmaxf(x, -80.f) * -1.44269504088896341f);
+  return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, EI_WAVE);

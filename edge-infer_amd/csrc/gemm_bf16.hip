@@ -41,10 +41,15 @@ __device__ __forceinline__ const bf16_t* packed_piece(const bf16_t* Wp, int n_st
 // outstanding is the same on every path and each wait leaves the younger loads in flight.
 // Few K slices: for many rows the float32 partial sums (rows x N x 4 bytes a slice, written
 // in 64-byte pieces and read again by the consumer) cost more than the weights they save.
-template <int MB, int WAVES, bool PACKED>
+//
+// GATED (one K slice only): the strips of W alternate between 16 gate rows and the 16 up rows
+// that belong to them; even waves hold gate sums, their odd neighbours the up sums, and the
+// block writes silu(gate) * up as bfloat16 [M, N/2] to `gated_out` instead of any sums.
+template <int MB, int WAVES, bool PACKED, bool GATED>
 __global__ void __launch_bounds__(WAVES * EI_WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
-                   float* __restrict__ out, int M, int N, int K, int k_per_split) {
+                   float* __restrict__ out, bf16_t* __restrict__ gated_out, int M, int N, int K,
+                   int k_per_split) {
   constexpr int KT = 256, JN = KT / 32;   // MFMA steps per K-tile
   constexpr int THREADS = WAVES * EI_WAVE;
   constexpr int ROWS_X = MB * 16;
@@ -187,6 +192,39 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
     }
   }
 
+  if (GATED) {
+    static_assert(!GATED || WAVES % 2 == 0, "gate and up strips are held by neighbouring waves");
+    // up sums travel through LDS (the X tiles are done with) to the wave that holds the gates
+    __syncthreads();
+    f32x4* exchange = reinterpret_cast<f32x4*>(&xs[0][0]);      // WAVES/2 * MB * 64 * 16 bytes
+    static_assert(sizeof(xs) >= WAVES / 2 * MB * EI_WAVE * sizeof(f32x4), "exchange fits");
+    if (wave & 1) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) exchange[((wave >> 1) * MB + mb) * EI_WAVE + lane] = acc[mb];
+    }
+    __syncthreads();
+    if (!(wave & 1) && n_tile + 16 < N) {
+      const int half = N / 2;
+      const int col = n_tile / 2 + 4 * c;                       // (strip / 2) * 16 + 4c
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int m = mb * 16 + r16;
+        if (m >= M) continue;
+        const f32x4 up = exchange[((wave >> 1) * MB + mb) * EI_WAVE + lane];
+        uint32_t packed[2];
+#pragma unroll
+        for (int r = 0; r < 4; r += 2) {
+          const bf16_t lo = ei::f32_to_bf16(ei::silu<bf16_t>(acc[mb][r]) * up[r]);
+          const bf16_t hi = ei::f32_to_bf16(ei::silu<bf16_t>(acc[mb][r + 1]) * up[r + 1]);
+          packed[r / 2] = static_cast<uint32_t>(lo) | (static_cast<uint32_t>(hi) << 16);
+        }
+        *reinterpret_cast<uint2*>(gated_out + static_cast<size_t>(m) * half + col) =
+            uint2{packed[0], packed[1]};
+      }
+    }
+    return;
+  }
+
   // lane (c, r16) holds out[m = mb*16 + r16][n_tile + 4c + 0..3]
   float* dst = out + static_cast<size_t>(blockIdx.y) * M * N;
   const int n0 = n_tile + 4 * c;
@@ -266,30 +304,38 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int max_splits) {
 
 namespace {
 
-template <int MB, bool PACKED>
-void launch_tile_kernel(const bf16_t* w, const bf16_t* x, float* out, int M, int N, int K,
-                        int k_per_split, int splits, hipStream_t stream) {
+template <int MB, bool PACKED, bool GATED>
+void launch_tile_kernel(const bf16_t* w, const bf16_t* x, float* out, bf16_t* gated_out, int M,
+                        int N, int K, int k_per_split, int splits, hipStream_t stream) {
   const int n_strips = (N + 15) / 16;
   const int waves = tile_kernel_waves(n_strips, splits, k_per_split / static_cast<double>(kTile), nullptr);
   dim3 grid((n_strips + waves - 1) / waves, splits);
   if (waves == 4)
-    skinny_gemm_kernel<MB, 4, PACKED><<<grid, 4 * EI_WAVE, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<MB, 4, PACKED, GATED><<<grid, 4 * EI_WAVE, 0, stream>>>(
+        w, x, out, gated_out, M, N, K, k_per_split);
   else if (waves == 6)
-    skinny_gemm_kernel<MB, 6, PACKED><<<grid, 6 * EI_WAVE, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<MB, 6, PACKED, GATED><<<grid, 6 * EI_WAVE, 0, stream>>>(
+        w, x, out, gated_out, M, N, K, k_per_split);
   else
-    skinny_gemm_kernel<MB, 8, PACKED><<<grid, 8 * EI_WAVE, 0, stream>>>(w, x, out, M, N, K, k_per_split);
+    skinny_gemm_kernel<MB, 8, PACKED, GATED><<<grid, 8 * EI_WAVE, 0, stream>>>(
+        w, x, out, gated_out, M, N, K, k_per_split);
 }
 
-template <bool PACKED>
-int launch_skinny(const void* X, const void* W, float* out, int M, int N, int K, int splits,
-                  hipStream_t stream) {
+template <bool PACKED, bool GATED>
+int launch_skinny(const void* X, const void* W, float* out, void* gated_out, int M, int N, int K,
+                  int splits, hipStream_t stream) {
   EI_REQUIRE(M >= 1 && M <= 64, "gemm_bf16_skinny: rows must lie in 1..64");
   EI_REQUIRE(N >= 1 && K >= 8 && K % 8 == 0, "gemm_bf16_skinny: K must be a multiple of 8");
-  EI_REQUIRE(X && W && out, "gemm_bf16_skinny: null pointer");
+  EI_REQUIRE(X && W && (GATED ? gated_out != nullptr : out != nullptr), "gemm_bf16_skinny: null pointer");
 
   EI_REQUIRE((reinterpret_cast<uintptr_t>(X) & 15) == 0 && (reinterpret_cast<uintptr_t>(W) & 15) == 0 &&
-                 (reinterpret_cast<uintptr_t>(out) & 15) == 0,
+                 (reinterpret_cast<uintptr_t>(out) & 15) == 0 &&
+                 (reinterpret_cast<uintptr_t>(gated_out) & 15) == 0,
              "gemm_bf16_skinny: pointers must be 16-byte aligned");
+  if (GATED) {
+    EI_REQUIRE(splits == 1, "gemm_bf16_skinny_gated: K cannot be sliced");
+    EI_REQUIRE(N % 32 == 0, "gemm_bf16_skinny_gated: N must be a multiple of 32 (gate and up strips)");
+  }
   const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   const int k_tiles = (K + kTile - 1) / kTile;
   EI_REQUIRE(splits >= 1 && splits <= k_tiles, "gemm_bf16_skinny: bad slice count");
@@ -297,12 +343,13 @@ int launch_skinny(const void* X, const void* W, float* out, int M, int N, int K,
   const int k_per_split = (k_tiles + splits - 1) / splits * kTile;
   const bf16_t* x = static_cast<const bf16_t*>(X);
   const bf16_t* w = static_cast<const bf16_t*>(W);
+  bf16_t* g = static_cast<bf16_t*>(gated_out);
   if (MB == 1) {
-    launch_tile_kernel<1, PACKED>(w, x, out, M, N, K, k_per_split, splits, stream);
+    launch_tile_kernel<1, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
   } else if (MB == 2) {
-    launch_tile_kernel<2, PACKED>(w, x, out, M, N, K, k_per_split, splits, stream);
+    launch_tile_kernel<2, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
   } else {
-    launch_tile_kernel<4, PACKED>(w, x, out, M, N, K, k_per_split, splits, stream);
+    launch_tile_kernel<4, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
   }
   EI_LAUNCH_CHECK();
 }
@@ -313,7 +360,7 @@ int launch_skinny(const void* X, const void* W, float* out, int M, int N, int K,
 // sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 64.
 extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int M, int N, int K,
                                    int splits, hipStream_t stream) {
-  return launch_skinny<false>(X, W, out, M, N, K, splits, stream);
+  return launch_skinny<false, false>(X, W, out, nullptr, M, N, K, splits, stream);
 }
 
 // The same product with W in the streaming layout: tiles of 16 rows x 32 k (1 KB each, rows
@@ -325,5 +372,15 @@ extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int
 // memory channel busy; rows of W that are 2^n bytes apart do not.
 extern "C" int ei_gemm_bf16_skinny_packed(const void* X, const void* Wp, float* out, int M, int N,
                                           int K, int splits, hipStream_t stream) {
-  return launch_skinny<true>(X, Wp, out, M, N, K, splits, stream);
+  return launch_skinny<true, false>(X, Wp, out, nullptr, M, N, K, splits, stream);
+}
+
+// Gated feed-forward in one pass: W [N, K] holds, in strips of 16 rows, the gate rows of 16
+// outputs followed by their up rows (N = 2 * outputs, a multiple of 32); act [M, N/2]
+// bfloat16 = silu(X . gate^T) * (X . up^T).  All of K in one slice.  `packed`: W is in the
+// streaming layout of ei_gemm_bf16_skinny_packed.
+extern "C" int ei_gemm_bf16_skinny_gated(const void* X, const void* W, void* act, int M, int N,
+                                         int K, int packed, hipStream_t stream) {
+  if (packed) return launch_skinny<true, true>(X, W, nullptr, act, M, N, K, 1, stream);
+  return launch_skinny<false, true>(X, W, nullptr, act, M, N, K, 1, stream);
 }

@@ -26,7 +26,7 @@ _SIGNATURES = {
         "ei_embed_gather": [c_void_p, c_void_p, c_int, c_void_p, c_int, c_int, c_int, c_void_p],
         "ei_add_rmsnorm": [c_void_p, c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p,
                            c_float, c_void_p, c_int, c_int, c_int, c_int, c_void_p],
-        "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int,
+        "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int, c_int,
                       c_void_p],
         "ei_sum_slices": [c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
     },
@@ -63,6 +63,8 @@ _SIGNATURES = {
                                 c_void_p],
         "ei_gemm_bf16_skinny_packed": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                                        c_void_p],
+        "ei_gemm_bf16_skinny_gated": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                      c_void_p],
     },
     "sampling": {
         "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
@@ -179,12 +181,15 @@ def add_rmsnorm(residual: torch.Tensor, delta: Optional[torch.Tensor], weight: t
     _check(lib, status, "add_rmsnorm")
 
 
-def swiglu(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+def swiglu(gate_up: torch.Tensor, out: torch.Tensor, strip: int = 0) -> None:
+    """out = silu(gate) * up of [n, 2*inter] rows (or float32 slices of them).  strip = 0:
+    the gate columns come first, then the up columns; strip > 0: `strip` gate columns,
+    their `strip` up columns, and so on."""
     lib = library("rowwise")
     n, inter = out.shape
     nsplit, stride = _splits(gate_up, n, 2 * inter, "gate_up")
     status = lib.ei_swiglu(_gpu(gate_up, "gate_up"), _code(gate_up, "gate_up"), nsplit, stride,
-                           _gpu(out, "out"), _code(out, "out"), n, inter, _stream())
+                           _gpu(out, "out"), _code(out, "out"), n, inter, int(strip), _stream())
     _check(lib, status, "swiglu")
 
 
@@ -460,3 +465,26 @@ def gemm_bf16_skinny_packed(x: torch.Tensor, packed: torch.Tensor, n: int,
                                             _gpu(out, "out", torch.float32), m, n, k,
                                             out.shape[0], _stream())
     _check(lib, status, "gemm_bf16_skinny_packed")
+
+
+GATE_STRIP = 16     # gate rows and up rows alternate in strips of this many (one MFMA tile)
+
+
+def gemm_bf16_skinny_gated(x: torch.Tensor, w: torch.Tensor, n: int, act: torch.Tensor,
+                           packed: bool) -> None:
+    """act[m, i] = silu(x[m] . gate_i) * (x[m] . up_i) for a weight [n, k] whose rows are, in
+    strips of 16, the gate rows of 16 outputs followed by their up rows; `w` is that matrix or
+    (packed) its `pack_weight` copy.  For at most 64 rows; K is not sliced, so it pays where
+    `skinny_gemm_splits` is 1."""
+    lib = library("gemm_bf16")
+    m, k = x.shape
+    if tuple(act.shape) != (m, n // 2) or n % (2 * GATE_STRIP):
+        raise KernelError(f"gemm_bf16_skinny_gated: {list(x.shape)} x [{n}, {k}] -> "
+                          f"{list(act.shape)} do not agree")
+    expect = (8 * ((k + 255) // 256), (n + 15) // 16, 4, 16, 8) if packed else (n, k)
+    if tuple(w.shape) != expect:
+        raise KernelError(f"gemm_bf16_skinny_gated: weight {list(w.shape)}, expected {list(expect)}")
+    status = lib.ei_gemm_bf16_skinny_gated(_gpu(x, "x", torch.bfloat16), _gpu(w, "w", torch.bfloat16),
+                                           _gpu(act, "act", torch.bfloat16), m, n, k, int(packed),
+                                           _stream())
+    _check(lib, status, "gemm_bf16_skinny_gated")

@@ -131,46 +131,43 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
   }
 }
 
+// Where gate and up of output column `col` lie in a row of 2I: the halves [gate | up]
+// (strip = 0), or strips of `strip` gate columns followed by their `strip` up columns.
+__device__ __forceinline__ size_t gate_column(size_t col, int strip) {
+  return strip ? (col / strip) * 2 * strip + col % strip : col;
+}
+
 template <typename TI, typename TO>
 __global__ void swiglu_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
-                              TO* __restrict__ out, int I, size_t total) {
+                              TO* __restrict__ out, int I, size_t total, int strip) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  const size_t up_offset = strip ? strip : I;
   for (size_t idx = start; idx < total; idx += step) {
     const size_t row = idx / I, col = idx % I;
-    const TI* g = gate_up + row * 2 * I + col;
+    const TI* g = gate_up + row * 2 * I + gate_column(col, strip);
     float gate = 0.f, up = 0.f;
     for (int s = 0; s < nsplit; ++s) {
       gate += ei::to_f32<TI>(g[s * split_stride]);
-      up += ei::to_f32<TI>(g[s * split_stride + I]);
+      up += ei::to_f32<TI>(g[s * split_stride + up_offset]);
     }
-    const float act = gate / (1.0f + expf(-gate));
-    out[idx] = ei::from_f32<TO>(act * up);
+    out[idx] = ei::from_f32<TO>(ei::silu<TO>(gate) * up);
   }
-}
-
-// x / (1 + e^-x).  For a float32 result the library's exponential and a true division;
-// for a bfloat16 result (8 bits of mantissa) the hardware's exp2 and reciprocal, both good
-// to about one unit in the 23rd bit, which the rounding to bfloat16 swallows.
-template <typename TO> __device__ __forceinline__ float silu(float x);
-template <> __device__ __forceinline__ float silu<float>(float x) { return x / (1.0f + expf(-x)); }
-template <> __device__ __forceinline__ float silu<bf16_t>(float x) {
-  const float e = __builtin_amdgcn_exp2f(fmaxf(x, -80.f) * -1.44269504088896341f);
-  return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
 // The same for I a multiple of 8: a thread takes 8 neighbouring columns of one row with
 // 16-byte (bfloat16) or 2 x 16-byte (float32) accesses.
 template <typename TI, typename TO>
 __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, size_t split_stride,
-                                  TO* __restrict__ out, int I, size_t total_octets) {
+                                  TO* __restrict__ out, int I, size_t total_octets, int strip) {
   const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
   const int octets_per_row = I / 8;
   for (size_t idx = start; idx < total_octets; idx += step) {
     const size_t row = idx / octets_per_row;
     const int col = static_cast<int>(idx % octets_per_row) * 8;
-    const TI* g = gate_up + row * 2 * I + col;
+    const TI* g = gate_up + row * 2 * I + gate_column(col, strip);   // strips hold whole octets
+    const size_t up_offset = strip ? strip : I;
     float gate[8], up[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) gate[i] = up[i] = 0.f;
@@ -182,8 +179,8 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
           const TI* p = g + (s0 + u) * split_stride;
           Vec4<TI>::load(p, a[u]);
           Vec4<TI>::load(p + 4, b[u]);
-          Vec4<TI>::load(p + I, c[u]);
-          Vec4<TI>::load(p + I + 4, d[u]);
+          Vec4<TI>::load(p + up_offset, c[u]);
+          Vec4<TI>::load(p + up_offset + 4, d[u]);
         }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -200,8 +197,8 @@ __global__ void swiglu_vec_kernel(const TI* __restrict__ gate_up, int nsplit, si
     float y0[4], y1[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      y0[i] = silu<TO>(gate[i]) * up[i];
-      y1[i] = silu<TO>(gate[i + 4]) * up[i + 4];
+      y0[i] = ei::silu<TO>(gate[i]) * up[i];
+      y1[i] = ei::silu<TO>(gate[i + 4]) * up[i + 4];
     }
     TO* dst = out + row * I + col;
     Vec4<TO>::store(dst, y0);
@@ -318,27 +315,29 @@ extern "C" int ei_add_rmsnorm(float* residual, const void* delta, int delta_dtyp
   EI_LAUNCH_CHECK();
 }
 
-// gate_up: [nsplit][N, 2I] (gate columns first), out: [N, I].
+// gate_up: [nsplit][N, 2I], out: [N, I].  strip = 0: gate columns first, then up columns;
+// strip > 0 (a divisor of I): `strip` gate columns, their `strip` up columns, and so on.
 extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long long split_stride,
-                         void* out, int out_dtype, int N, int I, hipStream_t stream) {
+                         void* out, int out_dtype, int N, int I, int strip, hipStream_t stream) {
   EI_REQUIRE(N > 0 && I > 0 && nsplit >= 1, "swiglu: sizes must be positive");
   EI_REQUIRE(gate_up && out, "swiglu: null pointer");
+  EI_REQUIRE(strip >= 0 && (strip == 0 || I % strip == 0), "swiglu: the strip must divide the width");
   const size_t total = static_cast<size_t>(N) * I;
   const int threads = 256;
   const size_t ss = static_cast<size_t>(split_stride);
-  if (I % 8 == 0 && ss % 8 == 0) {
+  if (I % 8 == 0 && ss % 8 == 0 && strip % 8 == 0) {
     const size_t octets = total / 8;
     size_t vblocks = (octets + threads - 1) / threads;
     if (vblocks > 256 * 32) vblocks = 256 * 32;
     if (in_dtype == EI_F32 && out_dtype == EI_F32)
       swiglu_vec_kernel<float, float><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip);
     else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
       swiglu_vec_kernel<float, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets);
+          static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip);
     else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
       swiglu_vec_kernel<bf16_t, bf16_t><<<vblocks, threads, 0, stream>>>(
-          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets);
+          static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, octets, strip);
     else
       EI_REQUIRE(false, "swiglu: unsupported dtype combination");
     EI_LAUNCH_CHECK();
@@ -347,13 +346,13 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
   if (blocks > 256 * 32) blocks = 256 * 32;
   if (in_dtype == EI_F32 && out_dtype == EI_F32)
     swiglu_kernel<float, float><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
     swiglu_kernel<float, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total);
+        static_cast<const float*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip);
   else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
     swiglu_kernel<bf16_t, bf16_t><<<blocks, threads, 0, stream>>>(
-        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total);
+        static_cast<const bf16_t*>(gate_up), nsplit, ss, static_cast<bf16_t*>(out), I, total, strip);
   else
     EI_REQUIRE(false, "swiglu: unsupported dtype combination");
   EI_LAUNCH_CHECK();

@@ -60,6 +60,23 @@ class Linear:
         torch.matmul(x, self.weight.t(), out=out)
         return out
 
+    def forward_gated(self, ctx, x: torch.Tensor, out_name: str):
+        """For a weight whose rows alternate, in strips of `lib.GATE_STRIP`, between gate rows
+        and their up rows: silu(gate) * up as [N, out/2] of the storage type straight from
+        the few-rows kernel, or None where that kernel does not apply (float32, many rows, a
+        shape whose K it would slice); the caller then takes `forward` and the activation
+        kernel."""
+        rows = x.shape[0]
+        if (self.dtype != torch.bfloat16 or not lib.skinny_gemm_ok(rows, self.in_features)
+                or self.out_features % (2 * lib.GATE_STRIP)
+                or lib.skinny_gemm_splits(rows, self.out_features, self.in_features) != 1):
+            return None
+        act = ctx.buffer(out_name, (rows, self.out_features // 2), torch.bfloat16)
+        packed = self.packed is not None
+        lib.gemm_bf16_skinny_gated(x, self.packed if packed else self.weight, self.out_features,
+                                   act, packed)
+        return act
+
     def forward_f32(self, ctx, x: torch.Tensor, out_name: str) -> torch.Tensor:
         """Like forward, but one float32 [N, out] tensor (used for the logits)."""
         rows = x.shape[0]

@@ -1,7 +1,11 @@
 """Gated feed-forward: down(silu(gate(x)) * up(x)).
 
 runtime/include/execution/decoder.hpp:161-166 of the reference; gate and up are
-two checkpoint matrices that become one [2I, H] matrix when the part is built.
+two checkpoint matrices that become one [2I, H] matrix when the part is built: in strips
+of 16 rows, the gate rows of 16 outputs followed by their up rows (when I is a multiple of
+16; else all gate rows, then all up rows).  A wave of the few-rows kernel owns 16 rows, so
+neighbouring waves hold a strip's gate and up sums and the kernel can write
+silu(gate) * up itself; otherwise the activation kernel reads the same layout.
 """
 from __future__ import annotations
 
@@ -25,13 +29,23 @@ class GatedMLP:
         if spec.activation != "silu":
             raise ValueError(f"gated_mlp: activation '{spec.activation}' is not implemented")
         self.spec = spec
-        self.gate_up = Linear(torch.cat([params["gate_proj.weight"], params["up_proj.weight"]],
-                                        dim=0), dtype, device)
+        gate, up = params["gate_proj.weight"], params["up_proj.weight"]
+        inter = spec.intermediate_size
+        self.strip = lib.GATE_STRIP if inter % lib.GATE_STRIP == 0 else 0
+        if self.strip:
+            both = torch.stack([gate.reshape(inter // self.strip, self.strip, hidden),
+                                up.reshape(inter // self.strip, self.strip, hidden)], dim=1)
+            both = both.reshape(2 * inter, hidden)
+        else:
+            both = torch.cat([gate, up], dim=0)
+        self.gate_up = Linear(both, dtype, device)
         self.down = Linear(params["down_proj.weight"], dtype, device)
 
     def forward(self, ctx, x):
         n = x.shape[0]
-        gate_up = self.gate_up.forward(ctx, x, "mlp.gate_up")
-        act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
-        lib.swiglu(gate_up, act)
+        act = self.gate_up.forward_gated(ctx, x, "mlp.act") if self.strip else None
+        if act is None:
+            gate_up = self.gate_up.forward(ctx, x, "mlp.gate_up")
+            act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
+            lib.swiglu(gate_up, act, self.strip)
         return self.down.forward(ctx, act, "mlp.down")

@@ -106,6 +106,23 @@ def test_swiglu(lib, dtype, I):
         close(out, plain.swiglu(one.double().cpu()[:, :I], one.double().cpu()[:, I:]), dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("I,strip", [(208, 16), (96, 4), (4096 + 16, 16)])
+def test_swiglu_with_gate_and_up_in_strips(lib, dtype, I, strip):
+    """Rows laid out as `strip` gate columns, their `strip` up columns, and so on (the
+    layout the gated feed-forward gives its fused matrix)."""
+    N = 3
+    gate = torch.randn(2, N, I, device=DEV) * 3
+    up = torch.randn(2, N, I, device=DEV)
+    mixed = torch.stack([gate.reshape(2, N, I // strip, strip),
+                         up.reshape(2, N, I // strip, strip)], dim=3).reshape(2, N, 2 * I)
+    out = torch.empty(N, I, device=DEV, dtype=dtype)
+    lib.swiglu(mixed.contiguous(), out, strip)
+    close(out, plain.swiglu(gate.double().cpu().sum(0), up.double().cpu().sum(0)), dtype)
+    with pytest.raises(lib.KernelError, match="divide"):
+        lib.swiglu(mixed.contiguous(), out, 7)
+
+
 @pytest.mark.parametrize("shape", [(1, 381, 96), (5, 64, 200), (70, 130, 33), (130, 257, 512)])
 def test_gemm_f32(lib, shape):
     M, N, K = shape
@@ -562,6 +579,36 @@ def test_gemm_bf16_skinny(lib, M, N, K):
         single = torch.empty((chosen, 1, N), device=DEV)
         lib.gemm_bf16_skinny(x[M // 2:M // 2 + 1].contiguous(), w, single)
         assert torch.equal(single[:, 0], results[chosen][:, M // 2])
+
+
+@pytest.mark.parametrize("packed", [True, False])
+@pytest.mark.parametrize("M,I,K", [(1, 48, 256), (8, 1024, 512), (16, 16, 96), (33, 2048, 256),
+                                   (64, 208, 1000)])
+def test_gemm_bf16_skinny_gated(lib, M, I, K, packed):
+    """silu(x . gate) * (x . up) written by the few-rows kernel itself, from a weight whose
+    rows alternate between 16 gate rows and their 16 up rows (all of K in one slice, also
+    where the plain product would cut it)."""
+    torch.manual_seed(M + I)
+    x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
+    gate = (torch.randn(I, K, device=DEV) / math.sqrt(K) * 3).to(torch.bfloat16)
+    up = (torch.randn(I, K, device=DEV) / math.sqrt(K)).to(torch.bfloat16)
+    mixed = torch.stack([gate.reshape(I // 16, 16, K), up.reshape(I // 16, 16, K)],
+                        dim=1).reshape(2 * I, K).contiguous()
+    act = torch.full((M, I), float("nan"), device=DEV, dtype=torch.bfloat16)
+    lib.gemm_bf16_skinny_gated(x, lib.pack_weight(mixed) if packed else mixed, 2 * I, act, packed)
+    expected = plain.swiglu(plain.linear(x.cpu(), gate.cpu()), plain.linear(x.cpu(), up.cpu()))
+    close(act, expected, torch.bfloat16)
+
+
+def test_gemm_bf16_skinny_gated_refuses_what_it_cannot_run(lib):
+    from edge_infer_amd.csrc.lib import KernelError
+    x = torch.zeros(2, 64, device=DEV, dtype=torch.bfloat16)
+    w = torch.zeros(48, 64, device=DEV, dtype=torch.bfloat16)        # 48 is no multiple of 32
+    with pytest.raises(KernelError, match="do not agree"):
+        lib.gemm_bf16_skinny_gated(x, w, 48, torch.empty(2, 24, device=DEV, dtype=torch.bfloat16), False)
+    w = torch.zeros(64, 64, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="do not agree"):            # act of the wrong width
+        lib.gemm_bf16_skinny_gated(x, w, 64, torch.empty(2, 64, device=DEV, dtype=torch.bfloat16), False)
 
 
 def test_gemm_bf16_skinny_refuses_what_it_cannot_run(lib):
