@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+                    [--shape 8b|0.6b|32b] [--only decode|prefill] [--prompt P]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
@@ -25,13 +26,23 @@ PREFILL_TOKENS = 2048
 CONTEXT = 4096
 
 
-def model_config(layers):
+# name: (layers, hidden, heads, kv heads, head_dim, intermediate, tied embeddings)
+SHAPES = {
+    "8b": (36, 4096, 32, 8, 128, 12288, False),
+    "0.6b": (28, 1024, 16, 8, 128, 3072, True),
+    "32b": (64, 5120, 64, 8, 128, 25600, False),
+}
+
+
+def model_config(shape, layers):
     import edge_infer_amd as ei
-    return ei.Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=layers,
-                          num_attention_heads=32, num_key_value_heads=8, head_dim=128,
-                          intermediate_size=12288, max_position_embeddings=40960,
+    full, hidden, heads, kv_heads, head_dim, inter, tied = SHAPES[shape]
+    return ei.Qwen3Config(vocab_size=151936, hidden_size=hidden,
+                          num_hidden_layers=layers or full, num_attention_heads=heads,
+                          num_key_value_heads=kv_heads, head_dim=head_dim,
+                          intermediate_size=inter, max_position_embeddings=40960,
                           bos_token_id=151643, eos_token_id=151645, rms_norm_eps=1e-6,
-                          rope_theta=1e6, tie_word_embeddings=False)
+                          rope_theta=1e6, tie_word_embeddings=tied)
 
 
 def step_bytes(cfg, batch, context, itemsize):
@@ -58,7 +69,7 @@ def synthetic_prompts(cfg, batch, length, seed):
     return torch.randint(0, cfg.vocab_size, (batch, length), generator=g).tolist()
 
 
-def measure_decode(model, cfg, batch, steps, warmup):
+def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT):
     """(ms per step, mean context during the timed steps)."""
     import torch
     import edge_infer_amd as ei
@@ -67,9 +78,9 @@ def measure_decode(model, cfg, batch, steps, warmup):
                          max_seq_tokens=CONTEXT)
     sampler = Sampler(model.device)
     greedy = SamplingParams(temperature=0.0)
-    prompts = synthetic_prompts(cfg, batch, PROMPT, seed=100 + batch)
+    prompts = synthetic_prompts(cfg, batch, prompt, seed=100 + batch)
     slots = [session.begin() for _ in range(batch)]
-    logits = session.step([(s, p, [PROMPT - 1]) for s, p in zip(slots, prompts)], copy=False)
+    logits = session.step([(s, p, [prompt - 1]) for s, p in zip(slots, prompts)], copy=False)
     tokens = sampler(logits, greedy, [], [])
 
     def run(count):
@@ -84,7 +95,7 @@ def measure_decode(model, cfg, batch, steps, warmup):
     run(steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
-    context = PROMPT + warmup + (steps + 1) / 2
+    context = prompt + warmup + (steps + 1) / 2
     for s in slots:
         session.end(s)
     del session
@@ -118,8 +129,12 @@ def main():
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=36,
-                        help="layers of the model (36 is the full Qwen3-8B shape)")
+    parser.add_argument("--shape", choices=sorted(SHAPES), default="8b",
+                        help="layer sizes: Qwen3-8B (the default and the headline), 0.6B or 32B")
+    parser.add_argument("--layers", type=int, default=0,
+                        help="layers of the model (0: as many as the shape has)")
+    parser.add_argument("--prompt", type=int, default=PROMPT,
+                        help="prompt length before the timed decode steps (with --only decode)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--skip-points", action="store_true")
     parser.add_argument("--only", choices=["decode", "prefill"], default=None,
@@ -131,20 +146,27 @@ def main():
 
     import torch
     import edge_infer_amd as ei
-    cfg = model_config(args.layers)
+    cfg = model_config(args.shape, args.layers)
+    full_layers = SHAPES[args.shape][0]
     model = ei.random_model(cfg, seed=2, dtype=args.dtype)
     torch.cuda.synchronize()
     itemsize = 2 if args.dtype == "bfloat16" else 4
 
     if args.only == "decode":
-        ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
-        print(json.dumps({"only": "decode", "batch": args.batch, "ms_per_step": round(ms_step, 4),
+        ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup,
+                                          args.prompt)
+        rate = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9
+        print(json.dumps({"only": "decode", "shape": args.shape, "batch": args.batch,
+                          "ms_per_step": round(ms_step, 4),
                           "tokens_per_s": round(args.batch * 1000.0 / ms_step, 1),
-                          "context": round(context)}))
+                          "context": round(context), "GB/s": round(rate, 1)}))
         return 0
     if args.only == "prefill":
         prefill_ms = measure_prefill(model, cfg)
-        print(json.dumps({"only": "prefill", "tokens": PREFILL_TOKENS, "ms": round(prefill_ms, 3)}))
+        flops = prefill_flops(cfg, PREFILL_TOKENS)
+        print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": PREFILL_TOKENS,
+                          "ms": round(prefill_ms, 3),
+                          "TFLOP/s": round(flops / (prefill_ms * 1e-3) / 1e12, 1)}))
         return 0
     ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
     value = args.batch * 1000.0 / ms_step
@@ -158,19 +180,21 @@ def main():
             points[name] = round(batch * 1000.0 / ms, 1)
     from edge_infer_amd.csrc import lib
     record = {
-        "metric": "decode tokens/s, Qwen3-8B shape, batch 8 after 512-token prompts",
+        "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch} after "
+                  f"{PROMPT}-token prompts",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic token ids, seeded random weights N(0, 0.02)",
         "config": {
-            "model": "Qwen3-8B shape", "layers": args.layers, "layers_full_model": 36,
+            "model": f"Qwen3-{args.shape.upper()} shape", "layers": cfg.num_hidden_layers,
+            "layers_full_model": full_layers,
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads,
             "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_norm_eps,
-            "tie_word_embeddings": False, "global_batch": args.batch, "prompt_len": PROMPT,
+            "tie_word_embeddings": cfg.tie_word_embeddings, "global_batch": args.batch, "prompt_len": PROMPT,
             "context_capacity": CONTEXT, "seq_len": round(context), "parallelism": "single GPU",
             "kernels": "+".join(lib.loaded_libraries()),
         },
