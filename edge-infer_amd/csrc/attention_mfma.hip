@@ -119,8 +119,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
       sc[r] = visible ? s[r] * scale : -INFINITY;
       tile_max = fmaxf(tile_max, sc[r]);
     }
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, EI_WAVE));
-    tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, EI_WAVE));
+    tile_max = ei::rows_max(tile_max);
     const float m_new = fmaxf(m_run, tile_max);
     const float alpha = expf(m_run - m_new);
     float tile_sum = 0.f;
@@ -130,8 +129,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
       p_lds[wave][4 * c + r][r16] = p;
       tile_sum += p;
     }
-    tile_sum += __shfl_xor(tile_sum, 16, EI_WAVE);
-    tile_sum += __shfl_xor(tile_sum, 32, EI_WAVE);
+    tile_sum = ei::rows_sum(tile_sum);
     l_run = l_run * alpha + tile_sum;
     m_run = m_new;
     if (c == 0) alpha_lds[wave][r16] = alpha;
@@ -406,8 +404,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
         for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[kb][r]);
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16, EI_WAVE));
-      tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32, EI_WAVE));
+      tile_max = ei::rows_max(tile_max);
       // running maximum in units of log2 (raw score * scale * log2 e; the scale is positive)
       const float m_new = fmaxf(m_run[rt], tile_max * scale_log2);
       const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
@@ -423,8 +420,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
             p_reg[rt][ks][half * 4 + r] = static_cast<__bf16>(p);
           }
       }
-      tile_sum += __shfl_xor(tile_sum, 16, EI_WAVE);
-      tile_sum += __shfl_xor(tile_sum, 32, EI_WAVE);
+      tile_sum = ei::rows_sum(tile_sum);
       l_run[rt] = l_run[rt] * alpha + tile_sum;
       m_run[rt] = m_new;
       if (__any(alpha != 1.f)) {            // the maximum of some row of this tile has moved

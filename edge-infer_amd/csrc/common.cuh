@@ -83,6 +83,27 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// Reductions over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), every lane
+// getting the result.  gfx950's row-swap instructions do each step in the vector ALU: with
+// both operands holding x, v_permlane32_swap leaves (x of the lower half, x of the upper
+// half) in all lanes of the two registers, v_permlane16_swap the same for neighbouring rows;
+// a shuffle through LDS (ds_bpermute) costs an LDS round trip instead.
+typedef unsigned int ei_u32x2 __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ float rows_max(float x) {
+  ei_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
+  r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return fmaxf(__uint_as_float(r.x), __uint_as_float(r.y));
+}
+
+__device__ __forceinline__ float rows_sum(float x) {
+  ei_u32x2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  x = __uint_as_float(r.x) + __uint_as_float(r.y);
+  r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+
 // Sum over a block of `blockDim.x` threads (a multiple of 64, at most 1024).
 // `scratch` holds at least 16 floats.  Every thread gets the total.
 __device__ __forceinline__ float block_sum(float v, float* scratch) {

@@ -107,19 +107,27 @@ class DecoderModel:
         return limit
 
     def capture_safe(self) -> bool:
-        """Whether a decode step may be captured in a HIP graph: every linear layer must
-        take the hand-written kernel for few rows (library products may record memset
-        nodes, which are not replayed reliably), and every mixer must say it is safe."""
+        """Whether a decode step may be captured in a HIP graph: every block and every
+        part that a block holds (norms, mixer, feed-forward) must say so with
+        `capture_safe = True` (it launches nothing but capturable kernels and allocates
+        nothing per step; a part that does not say so is taken to be unsafe), and every
+        linear layer must take the hand-written kernel for few rows (library products may
+        record memset nodes, which are not replayed reliably)."""
         def linears(obj, depth=0):
             if isinstance(obj, Linear):
                 yield obj
             elif depth < 3 and hasattr(obj, "__dict__"):
                 for value in vars(obj).values():
                     yield from linears(value, depth + 1)
+        if not getattr(self.final_norm, "capture_safe", False):
+            return False
         for layer in self.layers:
-            mixer = getattr(layer, "mixer", None)
-            if mixer is not None and not getattr(mixer, "capture_safe", False):
+            if not getattr(layer, "capture_safe", False):
                 return False
+            for part in vars(layer).values():
+                if hasattr(part, "forward") or hasattr(part, "add_norm"):
+                    if not getattr(part, "capture_safe", False):
+                        return False
             for linear in linears(layer):
                 if linear.dtype == torch.bfloat16 and linear.in_features % 8:
                     return False

@@ -11,6 +11,7 @@ class PreNormBlock:
     norm) performs it while reading the row."""
 
     parts = ("norm1", "mixer", "norm2", "ffn")
+    capture_safe = True      # nothing of its own besides its parts' kernels
 
     @classmethod
     def parameters(cls, layer_spec, hidden):

@@ -17,6 +17,8 @@ from .linear import Linear
 
 
 class GatedMLP:
+    capture_safe = True      # only capturable kernels, no allocation per step
+
     @classmethod
     def parameters(cls, spec, hidden):
         return {

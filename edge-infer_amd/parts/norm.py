@@ -14,6 +14,8 @@ from ..weights.loader import ParamSpec
 
 
 class RMSNorm:
+    capture_safe = True      # only capturable kernels, no allocation per step
+
     @classmethod
     def parameters(cls, spec, width):
         return {"weight": ParamSpec((width,), init="norm")}
