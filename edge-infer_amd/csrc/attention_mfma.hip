@@ -212,9 +212,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   }
 }
 
-// Prefill: a block of four waves owns HB query heads of one kv group (HB = 4, 2 or 1, the
-// largest that divides the group) and 32 * (4 / HB) consecutive positions of one sequence;
-// a wave keeps 32 rows (two 16-row tiles) of one head as MFMA operands in registers and
+// Prefill: a block of eight waves owns HB query heads of one kv group (HB = 4, 2 or 1, the
+// largest that divides the group) and 16 * (8 / HB) consecutive positions of one sequence;
+// a wave keeps 16 rows of one head as MFMA operands in registers (few enough registers for
+// two waves per SIMD, so that one wave's softmax runs beside the other's products) and
 // walks the key pages of the sequence.  A page of keys goes to LDS as stored, a page of
 // values goes to LDS transposed ([d][key]), once for the whole block, so the heads of a
 // group share every byte that is fetched.  Scores are computed transposed (S^T = K Q^T):
@@ -226,30 +227,37 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
 // Blocks are numbered so that the blocks of one kv head fall on one XCD (the hardware deals
 // consecutive workgroups round-robin to its 8 XCDs): that head's keys and values then stay
 // in that XCD's L2.
-constexpr int kRowTiles = 2;     // 16-row tiles per wave
+constexpr int kRowTiles = 1;     // 16-row tiles per wave
+constexpr int kPrefillWaves = 8; // two waves per SIMD: one's softmax overlaps the other's products
+constexpr int kPrefillThreads = kPrefillWaves * EI_WAVE;
 
 template <int D, int HB>
-__global__ void __launch_bounds__(kThreads)
+__global__ void __launch_bounds__(kPrefillThreads, 4)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                     const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
                     const int32_t* __restrict__ item_row0, const int32_t* __restrict__ item_npos,
                     int n_items, const int32_t* __restrict__ row_pos,
                     const int32_t* __restrict__ page_table, int table_width,
-                    bf16_t* __restrict__ out, int nq, int nkv, int window, float scale) {
+                    bf16_t* __restrict__ out, int nq, int nkv, int window, float scale,
+                    int pair) {
   constexpr int DJ = D / 32;             // MFMA steps over d for the scores
   constexpr int DB = D / 16;             // 16-wide output blocks over d
   constexpr int KS = D + 8;              // LDS stride of a key row (elements)
-  constexpr int VS = EI_PAGE + 8;        // LDS stride of a transposed value row
-  constexpr int CI = D / 32;             // 16-byte chunks per thread per page (D/8 * 64 / 256)
-  constexpr int PW = kWaves / HB;        // waves along the positions
+  constexpr int VS = EI_PAGE + 4;        // LDS stride of a transposed value row (34 dwords)
+  constexpr int CI = D / 64;             // 16-byte chunks per thread per page (D/8 * 64 / 512)
+  constexpr int PW = kPrefillWaves / HB; // waves along the positions
   constexpr int RT = kRowTiles;
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[EI_PAGE * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[D * VS];
+  // two pages of keys and of (transposed) values alternate, so that a page costs one barrier
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds2[2][EI_PAGE * KS];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds2[2][D * VS];
 
   // block number -> (kv head, head block, item) with the kv head fixed per XCD
   const int G = nq / nkv;
   const int head_blocks = G / HB;
-  const int rests = n_items * head_blocks;
+  // pair: a block takes item u and then item n - 1 - u, i.e. (the items being ordered by
+  // length) a long one and a short one, so that every block walks about as many pages
+  const int units = pair ? (n_items + 1) / 2 : n_items;
+  const int rests = units * head_blocks;
   int g, rest;
   {
     const int id = blockIdx.x, x = id & 7, slot = id >> 3;
@@ -267,14 +275,20 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     }
   }
   if (rest >= rests) return;
-  const int item = rest / head_blocks, hb = rest % head_blocks;
-  const int seq = item_seq[item];
-  if (seq < 0) return;
-  const int row0 = item_row0[item], npos = item_npos[item];
+  const int unit = rest / head_blocks, hb = rest % head_blocks;
   const int t = threadIdx.x, wave = t / EI_WAVE, lane = t % EI_WAVE;
   const int r16 = lane & 15, c = lane >> 4;
   const int hw = wave % HB, pw = wave / HB;
   const int head = g * G + hb * HB + hw;
+  for (int pass = 0; pass <= pair; ++pass) {
+  const int item = pass == 0 ? unit : n_items - 1 - unit;
+  if (pass == 1) {
+    if (item == unit) break;              // the middle item of an odd count
+    __syncthreads();                      // the first item's last page has been read
+  }
+  const int seq = item_seq[item];
+  if (seq < 0) continue;
+  const int row0 = item_row0[item], npos = item_npos[item];
 
   // this lane's query rows (columns n of S^T), their positions, and the Q operands
   int pos_r[RT];
@@ -315,8 +329,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     for (int db = 0; db < DB; ++db) o_acc[rt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  // global -> register staging of a page: thread t takes key t/4, chunks (t%4) + 4*i
-  const int ld_key = t >> 2, ld_dc = t & 3;
+  // global -> register staging of a page: thread t takes key t/8, chunks (t%8) + 8*i
+  const int ld_key = t >> 3, ld_dc = t & 7;
   uint4 k_stage[CI], v_stage[CI];
   // The physical page of the page after next is looked up while the next page's data is
   // on its way, so that a page costs one trip to memory, not two in a row.
@@ -334,37 +348,61 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     const bool live = page_index * EI_PAGE + ld_key <= last_pos;   // later slots: stale bytes
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
-      const int dc = ld_dc + 4 * i;
+      const int dc = ld_dc + 8 * i;
       k_stage[i] = live ? *reinterpret_cast<const uint4*>(k_pages + base + dc * 8)
                         : uint4{0u, 0u, 0u, 0u};
       v_stage[i] = live ? *reinterpret_cast<const uint4*>(v_pages + base + dc * 8)
                         : uint4{0u, 0u, 0u, 0u};
     }
   };
-  auto store_page = [&]() {
+  auto store_page = [&](int buf) {
+    bf16_t* k_lds = k_lds2[buf];
+    bf16_t* v_lds = v_lds2[buf];
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
-      const int dc = ld_dc + 4 * i;
+      const int dc = ld_dc + 8 * i;
       *reinterpret_cast<uint4*>(&k_lds[ld_key * KS + dc * 8]) = k_stage[i];
+      // Values go to LDS transposed ([d][key]).  A lane holds 8 values of one key as 4
+      // dwords (d pairs); the lane 8 further in its row of 16 holds the same d of the next
+      // key (keys come in even/odd pairs), so after one exchange (a DPP rotation of the row
+      // by 8) the even-key lane owns the two keys of the even d of every pair and the odd-key
+      // lane those of the odd d: 4 dword stores a lane instead of 8 halfword stores.  The 8
+      // lanes of a key write rows 8 apart, which a row stride of 34 dwords would put on 4
+      // banks; the upper 4 lanes take their d pairs one step later, which doubles that.
       const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
+      uint32_t pw[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        pw[e] = __builtin_amdgcn_update_dpp(0u, w[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+      const bool odd_key = ld_key & 1;
+      const bool later = ld_dc & 4;
+      const uint32_t take = odd_key ? 0x03020706u : 0x05040100u;   // bytes of (partner, own)
+      const int column = ld_key & ~1;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        v_lds[(dc * 8 + 2 * e) * VS + ld_key] = static_cast<bf16_t>(w[e] & 0xffffu);
-        v_lds[(dc * 8 + 2 * e + 1) * VS + ld_key] = static_cast<bf16_t>(w[e] >> 16);
+        const int e2 = (e + 1) & 3;
+        const uint32_t own = later ? w[e2] : w[e];
+        const uint32_t other = later ? pw[e2] : pw[e];
+        const int pair_index = later ? e2 : e;
+        // even key: (own.lo, partner.lo) = d even of keys (k, k+1); odd key: (partner.hi, own.hi)
+        const uint32_t both = __builtin_amdgcn_perm(other, own, take);
+        const int d = dc * 8 + 2 * pair_index + (odd_key ? 1 : 0);
+        *reinterpret_cast<uint32_t*>(&v_lds[d * VS + column]) = both;
       }
     }
   };
 
+  // Page p is multiplied from LDS buffer p & 1 while page p + 1 (fetched a page ago) goes
+  // from registers into the other buffer and page p + 2 is requested; the barrier at the
+  // end of a page says both that the other buffer is complete and that this one is free.
   load_page(lo_page, lookup(lo_page));
-  int phys_next = lookup(lo_page + 1);
+  store_page(lo_page & 1);
+  load_page(lo_page + 1, lookup(lo_page + 1));    // zeros past the last page
+  int phys_next = lookup(lo_page + 2);
+  __syncthreads();
   for (int page = lo_page; page <= hi_page; ++page) {
-    __syncthreads();                      // the previous page's reads are done
-    store_page();
-    __syncthreads();
-    if (page < hi_page) {
-      load_page(page + 1, phys_next);
-      phys_next = lookup(page + 2);
-    }
+    const bf16_t* k_lds = k_lds2[page & 1];
+    const bf16_t* v_lds = v_lds2[page & 1];
     const int key_base = page * EI_PAGE;
 
     // pages that every row of this wave sees in full (all but the last one or two of a
@@ -450,6 +488,12 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
                                                                   o_acc[rt][db], 0, 0, 0);
       }
     }
+    if (page < hi_page) {
+      store_page((page + 1) & 1);
+      load_page(page + 2, phys_next);
+      phys_next = lookup(page + 3);
+      __syncthreads();
+    }
   }
 
   // lane (c, n) holds O[query row 4c + r][d = db*16 + n]
@@ -467,6 +511,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
         dst[db * 16 + r16] = ei::from_f32<bf16_t>(o_acc[rt][db][r] * inv);
     }
   }
+  }  // pass
 }
 
 // One wave per (row, head): o = sum_s o_s e^{m_s - m} / sum_s l_s e^{m_s - m}.
@@ -530,7 +575,7 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
 // Positions of one sequence that a prefill work item of this file holds for a group ratio.
 extern "C" int ei_attn_prefill_mfma_positions(int G) {
   const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
-  return 16 * kRowTiles * (kWaves / HB);
+  return 16 * kRowTiles * (kPrefillWaves / HB);
 }
 
 template <int D, int HB>
@@ -538,10 +583,10 @@ static void launch_prefill(int blocks, hipStream_t stream, const bf16_t* q, cons
                            const bf16_t* v, const int32_t* item_seq, const int32_t* item_row0,
                            const int32_t* item_npos, int n_items, const int32_t* row_pos,
                            const int32_t* page_table, int table_width, bf16_t* out, int nq,
-                           int nkv, int window, float scale) {
-  attn_prefill_kernel<D, HB><<<blocks, kThreads, 0, stream>>>(
+                           int nkv, int window, float scale, int pair) {
+  attn_prefill_kernel<D, HB><<<blocks, kPrefillThreads, 0, stream>>>(
       q, k, v, item_seq, item_row0, item_npos, n_items, row_pos, page_table, table_width, out,
-      nq, nkv, window, scale);
+      nq, nkv, window, scale, pair);
 }
 
 // q, out: [N, nq, D] bfloat16; items: (sequence, first packed row, positions), each holding
@@ -560,7 +605,12 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
   EI_REQUIRE(window >= 0, "attention_prefill: negative window");
   const int G = nq / nkv;
   const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
-  const long long rests = static_cast<long long>(n_items) * (G / HB);
+  // Enough blocks to fill the chip twice over: pair a long item with a short one per block
+  // (the caller orders the items by length, longest first), so that the blocks take about
+  // equally long; with fewer blocks the pairs would leave compute units empty.
+  const int pair = static_cast<long long>(n_items) * (G / HB) * nkv >= 2 * 256 ? 1 : 0;
+  const long long units = pair ? (n_items + 1) / 2 : n_items;
+  const long long rests = units * (G / HB);
   long long blocks;
   if (nkv % 8 == 0) blocks = rests * nkv;
   else if (8 % nkv == 0) blocks = (rests + 8 / nkv - 1) / (8 / nkv) * 8;
@@ -573,7 +623,7 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
 #define EI_PREFILL(DD, HH)                                                                    \
   launch_prefill<DD, HH>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq, item_row0,   \
                          item_npos, n_items, row_pos, page_table, table_width, oo, nq, nkv,   \
-                         window, scale)
+                         window, scale, pair)
   if (D == 64) {
     if (HB == 4) EI_PREFILL(64, 4); else if (HB == 2) EI_PREFILL(64, 2); else EI_PREFILL(64, 1);
   } else {

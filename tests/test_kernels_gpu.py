@@ -427,6 +427,15 @@ def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D):
     close(out, expected, torch.bfloat16)
 
 
+@pytest.mark.parametrize("counts", [[1041, 20], [1060]])
+def test_attention_prefill_on_the_matrix_cores_many_blocks(lib, counts):
+    """Enough work items (more than 512 blocks) for the kernel to give every block two of
+    them, the u-th and the u-th from the end; an odd and an even number of items."""
+    out, expected = run_attention(lib, torch.bfloat16, 64, 16, 64, starts=[0] * len(counts),
+                                  counts=counts, kernel="prefill_mfma", seed=5)
+    close(out, expected, torch.bfloat16)
+
+
 @pytest.mark.parametrize("window", [1, 7, 64, 100])
 def test_attention_prefill_on_the_matrix_cores_window_and_far_key(lib, window):
     nq, nkv, D, n = 8, 2, 128, 230
