@@ -249,8 +249,8 @@ constexpr int kComputeUnits = 256;        // MI355X
 // Waves per block (4, 6 or 8) and what the busiest compute unit then has to do, in strips:
 // `strips * splits` strip-slices are dealt out in blocks of `waves` strips.  Up to two blocks
 // per unit all run at once, so the unit with the most blocks sets the time; many more blocks
-// than that even out.  Every block also costs a start (about 3 strip-tiles).  Ties go to the
-// larger block, which shares a tile of X among more waves.
+// than that even out.  Every block also costs a start (about 3 strip-tiles).  Near ties go
+// to the larger block, which shares a tile of X among more waves.
 int tile_kernel_waves(int n_strips, int splits, double tiles_per_slice, double* cost_out) {
   int best = 8;
   double best_cost = 1e30;
@@ -260,7 +260,7 @@ int tile_kernel_waves(int n_strips, int splits, double tiles_per_slice, double* 
                                 ? static_cast<double>((static_cast<long long>(blocks) + kComputeUnits - 1) / kComputeUnits)
                                 : blocks / kComputeUnits + 0.25;
     const double cost = per_unit * (waves * tiles_per_slice + 3.0);
-    if (cost < best_cost - 1e-9) {
+    if (cost < best_cost * 0.97) {          // a smaller block must be clearly better
       best_cost = cost;
       best = waves;
     }

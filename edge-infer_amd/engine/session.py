@@ -16,6 +16,7 @@ import torch
 from ..cache.allocator import PAGE_TOKENS, CacheFull
 from ..cache.storage import CacheLayout, SessionCache
 from ..parts.base import StepContext, Workspace
+from ..parts.linear import SKINNY_ROWS
 from .batch import DeviceMeta, SeqStep, StepPlan
 
 
@@ -187,7 +188,10 @@ class Session:
         growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
         self.cache.check_growth(growth)          # raises before anything changes
         self.cache.grow(growth)
-        if self.graphs and all(seq.count == 1 for seq in seqs):
+        # batches beyond the few-rows product's reach multiply through the library, whose
+        # kernels are kept out of graphs
+        if (self.graphs and len(seqs) <= SKINNY_ROWS
+                and all(seq.count == 1 for seq in seqs)):
             logits = self._run_captured(seqs)
         else:
             plan = StepPlan(seqs, item_sizes=self._item_sizes)
