@@ -70,19 +70,6 @@ template <> __device__ __forceinline__ float silu<bf16_t>(float x) {
   return x * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1) v += __shfl_xor(v, offset, EI_WAVE);
-  return v;
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1)
-    v = fmaxf(v, __shfl_xor(v, offset, EI_WAVE));
-  return v;
-}
-
 // Reductions over the four 16-lane rows of a wave (lanes l, l^16, l^32, l^48), every lane
 // getting the result.  gfx950's row-swap instructions do each step in the vector ALU: with
 // both operands holding x, v_permlane32_swap leaves (x of the lower half, x of the upper
@@ -102,6 +89,24 @@ __device__ __forceinline__ float rows_sum(float x) {
   x = __uint_as_float(r.x) + __uint_as_float(r.y);
   r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
   return __uint_as_float(r.x) + __uint_as_float(r.y);
+}
+
+// Sum over the 64 lanes, every lane getting it.  The steps inside a row of 16 lanes are DPP
+// operand modifiers of vector adds (quad permutes, then mirrors of half rows and rows), the
+// two across rows are gfx950's row swaps; no step goes through LDS as a shuffle would.
+__device__ __forceinline__ float wave_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xb1, 0xf, 0xf, false));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4e, 0xf, 0xf, false));   // quad_perm [2,3,0,1]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x141, 0xf, 0xf, false));  // row_half_mirror
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x140, 0xf, 0xf, false));  // row_mirror
+  return rows_sum(v);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int offset = EI_WAVE / 2; offset > 0; offset >>= 1)
+    v = fmaxf(v, __shfl_xor(v, offset, EI_WAVE));
+  return v;
 }
 
 // Sum over a block of `blockDim.x` threads (a multiple of 64, at most 1024).

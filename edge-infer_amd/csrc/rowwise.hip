@@ -64,6 +64,10 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ residual, const TD* __res
 // registers, up to 1024 threads a row so that few rows still have many loads in flight.
 using ei::Vec4;
 
+#ifndef EI_NORM_FEW_ROWS_THREADS
+#define EI_NORM_FEW_ROWS_THREADS 1024   // threads a row when rows are few (a build-time knob)
+#endif
+
 template <typename TD, typename TO, bool HAS_DELTA, int CHUNKS>
 __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* __restrict__ delta,
                                        int nsplit, size_t split_stride,
@@ -81,6 +85,12 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
     return;
   }
   float* res = residual + static_cast<size_t>(src) * H;
+  float w[CHUNKS][4];                      // asked for first: it depends on nothing
+#pragma unroll
+  for (int k = 0; k < CHUNKS; ++k) {
+    const int qd = threadIdx.x + k * blockDim.x;
+    if (qd < quads) Vec4<float>::load(weight + qd * 4, w[k]);
+  }
   float x[CHUNKS][4];
   float sum = 0.f;
 #pragma unroll
@@ -110,12 +120,6 @@ __global__ void add_rmsnorm_vec_kernel(float* __restrict__ residual, const TD* _
 #pragma unroll
       for (int i = 0; i < 4; ++i) sum += x[k][i] * x[k][i];
     }
-  }
-  float w[CHUNKS][4];                      // fetched before the reduction, not after it
-#pragma unroll
-  for (int k = 0; k < CHUNKS; ++k) {
-    const int qd = threadIdx.x + k * blockDim.x;
-    if (qd < quads) Vec4<float>::load(weight + qd * 4, w[k]);
   }
   const float total = ei::block_sum(sum, scratch);
   const float inv = rsqrtf(total / static_cast<float>(H) + eps);
@@ -255,7 +259,7 @@ static void launch_add_rmsnorm(float* residual, const void* delta, int nsplit, s
     const int quads = H / 4;
     // few rows: up to 1024 threads a row, so that many loads are in flight; many rows: 256
     // threads a row, so that several rows share a compute unit and overlap their phases
-    const int most = N >= 512 && quads <= 4 * 256 ? 256 : 1024;
+    const int most = N >= 512 && quads <= 4 * 256 ? 256 : EI_NORM_FEW_ROWS_THREADS;
     int threads = (quads + EI_WAVE - 1) / EI_WAVE * EI_WAVE;
     if (threads > most) threads = most;
     const int chunks = (quads + threads - 1) / threads;      // 1..4 for H <= 16384
