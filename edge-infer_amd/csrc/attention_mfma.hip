@@ -27,9 +27,11 @@ constexpr float kLowest = -1.0e30f;
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
-// GB: query heads of the kv group handled by this block (1..16).
-template <int D, int GB>
-__global__ void __launch_bounds__(kThreads)
+// GB: query heads of the kv group handled by this block (1..16).  W: waves of the block, each
+// taking every W-th tile of 16 keys of the block's key range: 4 where sequences and slices
+// give many blocks, 16 where they give few (a short range then needs no slices at all).
+template <int D, int GB, int W>
+__global__ void __launch_bounds__(W * EI_WAVE)
 attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                    const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ row_pos,
                    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table,
@@ -40,10 +42,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   constexpr int LPR = D / 8;            // lanes that cover one value row with 16-byte loads
   constexpr int KPI = EI_WAVE / LPR;    // value rows per load instruction
   constexpr int VI = kTile / KPI;       // value load instructions per tile
-  __shared__ float p_lds[kWaves][kTile][16];
-  __shared__ float alpha_lds[kWaves][16];
-  __shared__ float m_lds[kWaves][16], l_lds[kWaves][16];
-  __shared__ float o_lds[kWaves][GB][D];
+  __shared__ float p_lds[W][kTile][16];
+  __shared__ float alpha_lds[W][16];
+  __shared__ float m_lds[W][16], l_lds[W][16];
+  __shared__ float o_lds[W][GB][D];
 
   const int row = blockIdx.x;                      // packed row = sequence index in decode
   const int g = blockIdx.y / head_blocks, hb = blockIdx.y % head_blocks;
@@ -87,7 +89,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
   const int ks = lane / LPR, dc = lane % LPR;       // value rows: key sub-index, 8-wide chunk
 
-  for (int tile = tile_begin + wave; tile < tile_end; tile += kWaves) {
+  for (int tile = tile_begin + wave; tile < tile_end; tile += W) {
     const int key0 = tile * kTile;
     const int phys = page_table[static_cast<size_t>(seq) * table_width + key0 / EI_PAGE];
     if (phys < 0) continue;                        // released by the window: all masked
@@ -185,14 +187,14 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   }
   __syncthreads();
   // merge the four waves: thread -> (head, d), strided
-  for (int idx = t; idx < heads_here * D; idx += kThreads) {
+  for (int idx = t; idx < heads_here * D; idx += (W * EI_WAVE)) {
     const int h = idx / D, d = idx % D;
     float m = kLowest;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) m = fmaxf(m, m_lds[w][h]);
+    for (int w = 0; w < W; ++w) m = fmaxf(m, m_lds[w][h]);
     float l = 0.f, o = 0.f;
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
+    for (int w = 0; w < W; ++w) {
       const float f = expf(m_lds[w][h] - m);
       l += l_lds[w][h] * f;
       o += o_lds[w][h][d] * f;
@@ -564,10 +566,18 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
                    const bf16_t* v, const int32_t* row_pos, const int32_t* row_seq,
                    const int32_t* page_table, int table_width, bf16_t* out, float* part_o,
                    float* part_ml, int nq, int nkv, int head_blocks, int window, float scale,
-                   int n_splits) {
-  attn_decode_kernel<D, GB><<<grid, kThreads, 0, stream>>>(
-      q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-      head_blocks, window, scale, n_splits);
+                   int n_splits, int waves) {
+  if constexpr (GB <= 4) {               // larger head blocks: the merge buffers of 16 waves
+    if (waves == 16) {                   // would not fit in LDS
+      attn_decode_kernel<D, GB, 16><<<grid, 16 * EI_WAVE, 0, stream>>>(
+          q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
+          head_blocks, window, scale, n_splits);
+      return;
+    }
+  }
+  attn_decode_kernel<D, GB, 4><<<grid, 4 * EI_WAVE, 0, stream>>>(
+        q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
+        head_blocks, window, scale, n_splits);
 }
 
 }  // namespace
@@ -646,8 +656,9 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
                                         const int32_t* page_table, int table_width, void* out,
                                         float* part_o, float* part_ml, int rows, int nq, int nkv,
                                         int D, int window, float scale, int n_splits,
-                                        hipStream_t stream) {
+                                        int waves, hipStream_t stream) {
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
+  EI_REQUIRE(waves == 4 || waves == 16, "attention_decode: a block has 4 or 16 waves");
   EI_REQUIRE(D == 64 || D == 128, "attention_decode: this kernel takes head_dim 64 or 128");
   EI_REQUIRE(q && k_pages && v_pages && row_pos && row_seq && page_table && out && table_width > 0,
              "attention_decode: null pointer");
@@ -665,7 +676,8 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
   bf16_t* oo = static_cast<bf16_t*>(out);
 #define EI_DECODE(DD, GG)                                                                     \
   launch_decode<DD, GG>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table, table_width,  \
-                        oo, part_o, part_ml, nq, nkv, head_blocks, window, scale, n_splits)
+                        oo, part_o, part_ml, nq, nkv, head_blocks, window, scale, n_splits,   \
+                        waves)
 #define EI_DECODE_G(DD)            \
   switch (GB) {                    \
     case 1: EI_DECODE(DD, 1); break;   \

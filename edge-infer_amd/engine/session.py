@@ -37,6 +37,17 @@ class _Context(StepContext):
         wanted = (512 + blocks - 1) // blocks
         return max(1, min(wanted, pages, 32))
 
+    def decode_plan(self, n_kv_heads: int):
+        """(slices, waves per block) for the matrix-core decode kernel.  Few sequences with
+        contexts up to 2,048: one block of 16 waves per (sequence, kv head) takes the whole
+        key range, a tile of 16 keys per wave at a time, and nothing has to be merged
+        afterwards.  Otherwise blocks of 4 waves over slices of the range, as above (measured
+        faster for long contexts than fewer slices with more waves)."""
+        context = self._fixed_context or self.max_context
+        if self.n_seqs * n_kv_heads < 256 and context <= 2048:
+            return 1, 16
+        return self.decode_splits(n_kv_heads), 4
+
 
 class _CapturedDecode:
     """A decode step of a fixed batch size, captured once as a HIP graph.  Everything
@@ -78,7 +89,7 @@ class Session:
         # decode steps are replayed from HIP graphs unless the model has an operation
         # that is not safe to capture (see DecoderModel.capture_safe)
         self.graphs = bool(graphs) and model.capture_safe()
-        self._captured: Dict[int, _CapturedDecode] = {}
+        self._captured: Dict[Tuple[int, int], _CapturedDecode] = {}
         self.graph_replays = 0
 
     # -- slots -----------------------------------------------------------
@@ -215,18 +226,24 @@ class Session:
         return self.model.forward(self._context(plan, meta, workspace))
 
     def _run_captured(self, seqs: List[SeqStep]) -> torch.Tensor:
-        """A decode step through the graph of its batch-size bucket (powers of two).
-        The first step of a bucket runs eagerly on the bucket's own buffers and is then
-        captured; later steps only refresh the metadata and replay."""
+        """A decode step through the graph of its batch-size bucket (powers of two) and
+        context bound.  The first step of a bucket runs eagerly on the bucket's own buffers
+        and is then captured; later steps only refresh the metadata and replay."""
         live = len(seqs)
         bucket = 1
         while bucket < live:
             bucket *= 2
         plan = StepPlan(seqs, item_sizes=self._item_sizes, pad_seqs=bucket)
-        captured = self._captured.get(bucket)
+        # the launch shapes of attention depend on how long the sequences may be: a graph
+        # holds for contexts up to a bound (1,024, 4,096, ... or the capacity)
+        bound = 1024
+        while bound < plan.max_context:
+            bound *= 4
+        bound = min(bound, self.capacity)
+        captured = self._captured.get((bucket, bound))
         if captured is None:
-            captured = self._captured[bucket] = _CapturedDecode(self.device)
-        ctx = self._context(plan, captured.meta, captured.workspace, fixed_context=self.capacity)
+            captured = self._captured[(bucket, bound)] = _CapturedDecode(self.device)
+        ctx = self._context(plan, captured.meta, captured.workspace, fixed_context=bound)
         if captured.graph is None:
             logits = self.model.forward(ctx)
             torch.cuda.synchronize(self.device)

@@ -89,7 +89,8 @@ class Attention:
             spec.head_dim, write_cache=entry.writes_cache)
         out = ctx.buffer("attn.out", (n, spec.q_width))
         if ctx.decode:
-            splits = ctx.decode_splits(spec.n_kv_heads)
+            splits, waves = (ctx.decode_plan(spec.n_kv_heads) if self.matrix_cores
+                             else (ctx.decode_splits(spec.n_kv_heads), 4))
             part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
@@ -100,7 +101,8 @@ class Attention:
                 lib.attention_decode_mfma(q, k_pages, v_pages, meta.row_pos, meta.row_seq,
                                           page_table, out, spec.n_heads, spec.n_kv_heads,
                                           spec.head_dim, window=spec.window, scale=self.scale,
-                                          n_splits=splits, part_o=part_o, part_ml=part_ml)
+                                          n_splits=splits, part_o=part_o, part_ml=part_ml,
+                                          waves=waves)
             else:
                 item_seq, item_row0, item_npos, n_items = meta.decode_items()
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,

@@ -282,7 +282,7 @@ def items_for(lib, starts, counts, group, per=None):
 
 
 def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
-                  boost=None, kernel="generic"):
+                  boost=None, kernel="generic", waves=4):
     """Fill a paged cache with random keys and values, run the kernel for the last
     `counts[b]` positions of each sequence, return (kernel output, plain output)."""
     torch.manual_seed(seed)
@@ -321,7 +321,7 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     elif kernel == "decode_mfma":
         lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
                                   cache.table_dev, out, nq, nkv, D, window=window,
-                                  n_splits=splits, part_o=part_o, part_ml=part_ml)
+                                  n_splits=splits, part_o=part_o, part_ml=part_ml, waves=waves)
     else:
         lib.attention(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0, item_npos,
                       n_items, pos, seq, cache.table_dev, out, nq, nkv, D, window=window,
@@ -393,12 +393,15 @@ def test_attention_window_edge(lib, dtype, window):
 @pytest.mark.parametrize("nq,nkv,D,splits", [(32, 8, 128, 1), (32, 8, 128, 4), (8, 8, 64, 3),
                                              (6, 2, 128, 2), (20, 1, 64, 5), (16, 1, 128, 32),
                                              (2, 1, 64, 1)])
-def test_attention_decode_on_the_matrix_cores(lib, nq, nkv, D, splits):
+@pytest.mark.parametrize("waves", [4, 16])
+def test_attention_decode_on_the_matrix_cores(lib, nq, nkv, D, splits, waves):
     """The bfloat16 decode kernel: lengths around tile (16), page (64) and slice
-    boundaries, group ratios that fill a head block partly, more slices than pages."""
+    boundaries, group ratios that fill a head block partly, more slices than pages; blocks
+    of 4 and of 16 waves (more waves than a short sequence has tiles)."""
     starts = [0, 1, 14, 15, 16, 62, 63, 64, 127, 128, 300, 1029, 8]
     out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, starts=starts,
-                                  counts=[1] * len(starts), splits=splits, kernel="decode_mfma")
+                                  counts=[1] * len(starts), splits=splits, kernel="decode_mfma",
+                                  waves=waves)
     close(out, expected, torch.bfloat16)
 
 
@@ -408,7 +411,7 @@ def test_attention_decode_on_the_matrix_cores_window_and_far_key(lib, window):
     for key_index in (n - window, n - window - 1):
         out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [n - 1], [1], window=window,
                                       splits=3, boost=(0, key_index, 0, 300.0), seed=9,
-                                      kernel="decode_mfma")
+                                      kernel="decode_mfma", waves=16 if window > 7 else 4)
         close(out, expected, torch.bfloat16)
     out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [899], [1], splits=6,
                                   boost=(0, 3, 0, 200.0), seed=4, kernel="decode_mfma")
