@@ -49,19 +49,33 @@ template <int MB, int WAVES, bool PACKED, bool GATED>
 __global__ void __launch_bounds__(WAVES * EI_WAVE)
 skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
                    float* __restrict__ out, bf16_t* __restrict__ gated_out, int M, int N, int K,
-                   int k_per_split) {
+                   int k_per_split, int row_groups) {
   constexpr int KT = 256, JN = KT / 32;   // MFMA steps per K-tile
   constexpr int THREADS = WAVES * EI_WAVE;
   constexpr int ROWS_X = MB * 16;
-  constexpr int XS = KT + 8;              // LDS row stride in elements (16 bytes of padding)
-  constexpr int CHUNKS = ROWS_X * (KT / 8);
-  constexpr int XLOADS = (CHUNKS + THREADS - 1) / THREADS;
+  constexpr int XS = KT;                  // LDS row stride in elements; the 16-byte chunks of a
+                                          // row are stored at (chunk ^ row % 16), see store_x
+  // X travels in wave loads of two rows (2 x 512 bytes) each: lane (half, chunk) takes the
+  // 16-byte chunk `chunk` of row 2 * load + half
+  constexpr int PAIRS = ROWS_X / 2;
+  constexpr int XLOADS = (PAIRS + WAVES - 1) / WAVES;
   __shared__ __attribute__((aligned(16))) bf16_t xs[2][ROWS_X * XS];
 
   const int t = threadIdx.x;
-  const int wave = t / EI_WAVE, lane = t % EI_WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(t / EI_WAVE), lane = t % EI_WAVE;
   const int r16 = lane & 15, c = lane >> 4;
-  const int n_tile = (blockIdx.x * WAVES + wave) * 16;
+  // More than ROWS_X rows: `row_groups` blocks share every strip group, each with ROWS_X rows
+  // of X.  Block ids go round the 8 dies, so the blocks of one strip group are 8 ids apart:
+  // they start together on one die and the later ones find the weights in its L2.
+  int strip_block = blockIdx.x, row0 = 0;
+  if (row_groups > 1) {
+    row0 = (strip_block >> 3) % row_groups * ROWS_X;
+    strip_block = strip_block / (8 * row_groups) * 8 + (strip_block & 7);
+  }
+  if (strip_block * WAVES * 16 >= N || row0 >= M) return;
+  const int rows_here = min(ROWS_X, M - row0);
+  X += static_cast<size_t>(row0) * K;
+  const int n_tile = (strip_block * WAVES + wave) * 16;
   const int k_begin = blockIdx.y * k_per_split;
   const int k_end = min(K, k_begin + k_per_split);
   const int n_iter = (k_end - k_begin + KT - 1) / KT;
@@ -71,8 +85,10 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   if (w_row >= N) w_row = N - 1;          // rows past the end repeat the last one; never stored
   const int n_strips = (N + 15) / 16;
   const int strip = min(n_tile / 16, n_strips - 1);
-  const bf16_t* w_ptr = PACKED ? packed_piece(W, n_strips, 0, strip, lane)
-                               : W + static_cast<size_t>(w_row) * K + c * 8;
+  const bf16_t* w_ptr = W + static_cast<size_t>(w_row) * K + c * 8;     // stored layout
+  // packed: a base that is the same for the whole block plus a lane's 32-bit offset (the
+  // loads then take a scalar address and need no address registers)
+  const unsigned w_lane = (static_cast<unsigned>(strip) * kPackedTile + lane * 8) * 2u;  // bytes
   const size_t tile_stride = static_cast<size_t>(n_strips) * kPackedTile;
 
   f32x4 acc[MB];
@@ -87,34 +103,43 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
     const int kb = k_begin + tile * KT;
     if (PACKED) {
       // the packed copy holds whole K-tiles (zeros past K): no test
-      w[set][j] = __builtin_nontemporal_load(
-          reinterpret_cast<const bf16x8*>(w_ptr + (kb / 32 + j) * tile_stride));
+      const bf16_t* tile = W + (kb / 32 + j) * tile_stride;
+      w[set][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(
+          reinterpret_cast<const char*>(tile) + w_lane));
     } else {
       // clamped to the last piece of the slice; the matching piece of X is zero there
       const int k = min(kb + j * 32 + c * 8, k_end - 8);
       w[set][j] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w_ptr + k - c * 8));
     }
   };
+  // Rows past the last one repeat it (their sums are never stored), so every load is in
+  // bounds and none is conditional; k past the end of the slice can only occur in its last
+  // tile, where the address is clamped and zeros are stored instead.
+  const int x_half = lane >> 5, x_chunk = lane & 31;
+  unsigned x_row[XLOADS];
+#pragma unroll
+  for (int i = 0; i < XLOADS; ++i)
+    x_row[i] = static_cast<unsigned>(min(2 * (wave + i * WAVES) + x_half, rows_here - 1)) * K;
   auto load_x = [&](int tile) {
     const int kb = k_begin + tile * KT;
+    const unsigned k = min(kb + x_chunk * 8, k_end - 8);
 #pragma unroll
-    for (int i = 0; i < XLOADS; ++i) {
-      const int q = t + i * THREADS;
-      const int row = q / (KT / 8), k = kb + (q % (KT / 8)) * 8;
-      const bool valid = row < M && k < k_end;
-      x_regs[i] = *reinterpret_cast<const u32x4*>(
-          X + static_cast<size_t>(valid ? row : 0) * K + (valid ? k : k_begin));
-    }
+    for (int i = 0; i < XLOADS; ++i)
+      x_regs[i] = *reinterpret_cast<const u32x4*>(X + (x_row[i] + k));
   };
-  auto store_x = [&](int buf, int tile) {
-    const int kb = k_begin + tile * KT;
+  // `last_tag`: the tile may be the last of the slice (k is checked)
+  auto store_x = [&](int buf, int tile, auto last_tag) {
+    constexpr bool check_k = decltype(last_tag)::value;
+    const bool k_ok = !check_k || k_begin + tile * KT + x_chunk * 8 < k_end;
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
-      const int q = t + i * THREADS;
-      const int row = q / (KT / 8), ch = q % (KT / 8);
-      const bool valid = row < M && kb + ch * 8 < k_end;
-      if (CHUNKS % THREADS == 0 || q < CHUNKS)
-        *reinterpret_cast<u32x4*>(&xs[buf][row * XS + ch * 8]) = valid ? x_regs[i] : zero4;
+      const int pair = wave + i * WAVES;               // the same for the whole wave
+      const int row = 2 * pair + x_half;
+      // swizzled so that the operand reads below (16 rows, quarters c and c + 1 of a
+      // 32-wide step in one access group) touch every bank once
+      if (PAIRS % WAVES == 0 || pair < PAIRS)
+        *reinterpret_cast<u32x4*>(&xs[buf][row * XS + (x_chunk ^ (row & 15)) * 8]) =
+            k_ok ? x_regs[i] : zero4;
     }
   };
   // products of a tile whose W is in register set `set` and whose X is in LDS buffer `set`
@@ -123,18 +148,23 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   auto compute = [&](auto set_tag, auto refill_tag, int refill) {
     constexpr int set = decltype(set_tag)::value;
     constexpr bool do_refill = decltype(refill_tag)::value;
-    const bf16_t* x_base = &xs[set][r16 * XS + c * 8];
+    // chunk 4j + c of row r16 lies at chunk (4j + c) ^ r16 = 4 (j ^ r16 / 4) + (c ^ r16 % 4):
+    // four lane addresses (j % 4), the rest are constant offsets
+    const bf16_t* x_base = &xs[set][r16 * XS + (c ^ (r16 & 3)) * 8];
+    const bf16_t* x_step[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) x_step[jj] = x_base + (jj ^ (r16 >> 2)) * 32;
     bf16x8 xf[2][MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
-      xf[0][mb] = *reinterpret_cast<const bf16x8*>(x_base + mb * 16 * XS);
+      xf[0][mb] = *reinterpret_cast<const bf16x8*>(x_step[0] + mb * 16 * XS);
 #pragma unroll
     for (int j = 0; j < JN; ++j) {
       if (j + 1 < JN) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          xf[(j + 1) & 1][mb] =
-              *reinterpret_cast<const bf16x8*>(x_base + mb * 16 * XS + (j + 1) * 32);
+          xf[(j + 1) & 1][mb] = *reinterpret_cast<const bf16x8*>(
+              x_step[(j + 1) & 3] + mb * 16 * XS + ((j + 1) & 4) * 32);
       }
       // keep this order (reads of the next step, products, refill): left alone the
       // scheduler pairs every read with its use and gathers the refills at the end
@@ -154,39 +184,41 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   load_x(0);
 #pragma unroll
   for (int j = 0; j < JN; ++j) load_w_piece(0, 0, j);
+  using Inner = std::false_type;
+  using MaybeLast = std::true_type;
   if (n_iter == 1) {
-    store_x(0, 0);
+    store_x(0, 0, MaybeLast{});
     __syncthreads();
     compute(Set0{}, Last{}, 0);
   } else {
 #pragma unroll
     for (int j = 0; j < JN; ++j) load_w_piece(1, 1, j);
-    store_x(0, 0);
+    store_x(0, 0, Inner{});
     load_x(1);
     __syncthreads();
     int i = 0;                            // even: tile i is in set 0
     for (; i + 3 < n_iter; i += 2) {      // tiles i + 2 and i + 3 exist
       compute(Set0{}, Refill{}, i + 2);
-      store_x(1, i + 1);
+      store_x(1, i + 1, Inner{});
       load_x(i + 2);
       __syncthreads();
       compute(Set1{}, Refill{}, i + 3);
-      store_x(0, i + 2);
+      store_x(0, i + 2, Inner{});
       load_x(i + 3);
       __syncthreads();
     }
     if (i + 2 < n_iter) {                 // three tiles remain
       compute(Set0{}, Refill{}, i + 2);
-      store_x(1, i + 1);
+      store_x(1, i + 1, Inner{});
       load_x(i + 2);
       __syncthreads();
       compute(Set1{}, Last{}, 0);
-      store_x(0, i + 2);
+      store_x(0, i + 2, MaybeLast{});
       __syncthreads();
       compute(Set0{}, Last{}, 0);
     } else {                              // two
       compute(Set0{}, Last{}, 0);
-      store_x(1, i + 1);
+      store_x(1, i + 1, MaybeLast{});
       __syncthreads();
       compute(Set1{}, Last{}, 0);
     }
@@ -208,7 +240,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
       const int col = n_tile / 2 + 4 * c;                       // (strip / 2) * 16 + 4c
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        const int m = mb * 16 + r16;
+        const int m = row0 + mb * 16 + r16;
         if (m >= M) continue;
         const f32x4 up = exchange[((wave >> 1) * MB + mb) * EI_WAVE + lane];
         uint32_t packed[2];
@@ -230,7 +262,7 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   const int n0 = n_tile + 4 * c;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
-    const int m = mb * 16 + r16;
+    const int m = row0 + mb * 16 + r16;
     if (m >= M) continue;
     float* p = dst + static_cast<size_t>(m) * N + n0;
     if (n0 + 3 < N && (N & 3) == 0) {
@@ -245,17 +277,21 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
 
 constexpr int kTile = 256;                // K-tile of the kernel
 constexpr int kComputeUnits = 256;        // MI355X
+constexpr int kGroupRows = 64;            // rows of X one block takes
+constexpr int kMaxRows = 256;
 
 // Waves per block (4, 6 or 8) and what the busiest compute unit then has to do, in strips:
 // `strips * splits` strip-slices are dealt out in blocks of `waves` strips.  Up to two blocks
 // per unit all run at once, so the unit with the most blocks sets the time; many more blocks
 // than that even out.  Every block also costs a start (about 3 strip-tiles).  Near ties go
-// to the larger block, which shares a tile of X among more waves.
-int tile_kernel_waves(int n_strips, int splits, double tiles_per_slice, double* cost_out) {
+// to the larger block, which shares a tile of X among more waves.  `row_groups` blocks work
+// on every strip group (more than 64 rows of X).
+int tile_kernel_waves(int n_strips, int splits, int row_groups, double tiles_per_slice,
+                      double* cost_out) {
   int best = 8;
   double best_cost = 1e30;
   for (int waves = 8; waves >= 4; waves -= 2) {
-    const double blocks = static_cast<double>((n_strips + waves - 1) / waves) * splits;
+    const double blocks = static_cast<double>((n_strips + waves - 1) / waves) * splits * row_groups;
     const double per_unit = blocks <= 2 * kComputeUnits
                                 ? static_cast<double>((static_cast<long long>(blocks) + kComputeUnits - 1) / kComputeUnits)
                                 : blocks / kComputeUnits + 0.25;
@@ -292,7 +328,7 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int max_splits) {
     if (!valid_slice_count(k_tiles, splits)) continue;
     const double tiles = static_cast<double>((k_tiles + splits - 1) / splits);
     double cost = 0.0;                                   // in strip-tiles (8 KB of W) per unit
-    tile_kernel_waves(n_strips, splits, tiles, &cost);
+    tile_kernel_waves(n_strips, splits, (M + kGroupRows - 1) / kGroupRows, tiles, &cost);
     cost += 2.5 * splits * static_cast<double>(M) * N * 4.0 / kComputeUnits / 8192.0;
     if (cost < best_cost - 1e-9) {
       best_cost = cost;
@@ -308,23 +344,27 @@ template <int MB, bool PACKED, bool GATED>
 void launch_tile_kernel(const bf16_t* w, const bf16_t* x, float* out, bf16_t* gated_out, int M,
                         int N, int K, int k_per_split, int splits, hipStream_t stream) {
   const int n_strips = (N + 15) / 16;
-  const int waves = tile_kernel_waves(n_strips, splits, k_per_split / static_cast<double>(kTile), nullptr);
-  dim3 grid((n_strips + waves - 1) / waves, splits);
+  const int row_groups = (M + MB * 16 - 1) / (MB * 16);
+  const int waves = tile_kernel_waves(n_strips, splits, row_groups,
+                                      k_per_split / static_cast<double>(kTile), nullptr);
+  int strip_blocks = (n_strips + waves - 1) / waves;
+  if (row_groups > 1) strip_blocks = (strip_blocks + 7) / 8 * 8;   // whole rounds of the dies
+  dim3 grid(strip_blocks * row_groups, splits);
   if (waves == 4)
     skinny_gemm_kernel<MB, 4, PACKED, GATED><<<grid, 4 * EI_WAVE, 0, stream>>>(
-        w, x, out, gated_out, M, N, K, k_per_split);
+        w, x, out, gated_out, M, N, K, k_per_split, row_groups);
   else if (waves == 6)
     skinny_gemm_kernel<MB, 6, PACKED, GATED><<<grid, 6 * EI_WAVE, 0, stream>>>(
-        w, x, out, gated_out, M, N, K, k_per_split);
+        w, x, out, gated_out, M, N, K, k_per_split, row_groups);
   else
     skinny_gemm_kernel<MB, 8, PACKED, GATED><<<grid, 8 * EI_WAVE, 0, stream>>>(
-        w, x, out, gated_out, M, N, K, k_per_split);
+        w, x, out, gated_out, M, N, K, k_per_split, row_groups);
 }
 
 template <bool PACKED, bool GATED>
 int launch_skinny(const void* X, const void* W, float* out, void* gated_out, int M, int N, int K,
                   int splits, hipStream_t stream) {
-  EI_REQUIRE(M >= 1 && M <= 64, "gemm_bf16_skinny: rows must lie in 1..64");
+  EI_REQUIRE(M >= 1 && M <= kMaxRows, "gemm_bf16_skinny: rows must lie in 1..256");
   EI_REQUIRE(N >= 1 && K >= 8 && K % 8 == 0, "gemm_bf16_skinny: K must be a multiple of 8");
   EI_REQUIRE(X && W && (GATED ? gated_out != nullptr : out != nullptr), "gemm_bf16_skinny: null pointer");
 
@@ -357,7 +397,8 @@ int launch_skinny(const void* X, const void* W, float* out, void* gated_out, int
 }  // namespace
 
 // X: [M, K] bfloat16, W: [N, K] bfloat16, out: [splits, M, N] float32 (slice s holds the
-// sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 64.
+// sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 256
+// (beyond 64 rows, blocks of 64 rows each share the weights through the L2 of their die).
 extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int M, int N, int K,
                                    int splits, hipStream_t stream) {
   return launch_skinny<false, false>(X, W, out, nullptr, M, N, K, splits, stream);

@@ -417,13 +417,19 @@ def skinny_gemm_splits(rows: int, n: int, k: int) -> int:
     return library("gemm_bf16").ei_skinny_gemm_splits(rows, n, k, _SKINNY_MAX_SPLITS)
 
 
+# most rows for which the weight-streaming product is taken instead of the library's
+SKINNY_ROWS = int(os.environ.get("EDGE_INFER_SKINNY_ROWS", "128"))
+if not 1 <= SKINNY_ROWS <= 256:
+    raise KernelError("EDGE_INFER_SKINNY_ROWS must lie in 1..256")
+
+
 def skinny_gemm_ok(rows: int, k: int) -> bool:
-    return rows <= 64 and k % 8 == 0
+    return rows <= SKINNY_ROWS and k % 8 == 0
 
 
 def gemm_bf16_skinny(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
     """out[s, m, n] = sum over the s-th slice of K of x[m, :] . w[n, :] (float32), for at
-    most 64 rows; out.shape[0] says into how many slices K is cut."""
+    most 256 rows; out.shape[0] says into how many slices K is cut."""
     lib = library("gemm_bf16")
     m, k = x.shape
     n = w.shape[0]
@@ -476,7 +482,7 @@ def gemm_bf16_skinny_gated(x: torch.Tensor, w: torch.Tensor, n: int, act: torch.
                            packed: bool) -> None:
     """act[m, i] = silu(x[m] . gate_i) * (x[m] . up_i) for a weight [n, k] whose rows are, in
     strips of 16, the gate rows of 16 outputs followed by their up rows; `w` is that matrix or
-    (packed) its `pack_weight` copy.  For at most 64 rows; K is not sliced, so it pays where
+    (packed) its `pack_weight` copy.  For at most 256 rows; K is not sliced, so it pays where
     `skinny_gemm_splits` is 1."""
     lib = library("gemm_bf16")
     m, k = x.shape

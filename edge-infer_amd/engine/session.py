@@ -226,13 +226,15 @@ class Session:
         return self.model.forward(self._context(plan, meta, workspace))
 
     def _run_captured(self, seqs: List[SeqStep]) -> torch.Tensor:
-        """A decode step through the graph of its batch-size bucket (powers of two) and
-        context bound.  The first step of a bucket runs eagerly on the bucket's own buffers
+        """A decode step through the graph of its batch-size bucket (powers of two up to
+        64, then steps of 32) and context bound.  The first step of a bucket runs eagerly on the bucket's own buffers
         and is then captured; later steps only refresh the metadata and replay."""
         live = len(seqs)
         bucket = 1
-        while bucket < live:
+        while bucket < live and bucket < 64:
             bucket *= 2
+        if bucket < live:
+            bucket = (live + 31) // 32 * 32
         plan = StepPlan(seqs, item_sizes=self._item_sizes, pad_seqs=bucket)
         # the launch shapes of attention depend on how long the sequences may be: a graph
         # holds for contexts up to a bound (1,024, 4,096, ... or the capacity)

@@ -21,7 +21,7 @@ import torch
 
 from ..csrc import lib
 
-SKINNY_ROWS = 64
+SKINNY_ROWS = lib.SKINNY_ROWS
 STREAM_COPY = os.environ.get("EDGE_INFER_STREAM_COPY", "1") != "0"
 
 
@@ -84,7 +84,7 @@ class Linear:
         if self.dtype == torch.float32:
             lib.gemm_f32(x, self.weight, out)
             return out
-        if self.in_features % 8 == 0 and rows <= 4 * SKINNY_ROWS:
+        if self.in_features % 8 == 0 and rows <= max(256, SKINNY_ROWS):
             for start in range(0, rows, SKINNY_ROWS):
                 stop = min(rows, start + SKINNY_ROWS)
                 count = stop - start

@@ -156,6 +156,25 @@ def test_batch_composition_changes_nothing(models, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_batch_wider_than_64_sequences(models, oracle, dtype):
+    """70 short requests of 3 to 12 tokens start together and end one after another, so the
+    decode steps run with 70, then fewer and fewer rows: past 64 rows the few-rows product
+    works in groups of 64 rows (bfloat16), and every batch bucket on the way down is used."""
+    import edge_infer_amd as ei
+    name = "A"
+    cfg, w = oracle[name]
+    lengths = [3 + (7 * i) % 10 for i in range(70)]
+    requests = requests_for(name, lengths, seed=501)
+    session = ei.Session(models(name, dtype), max_tokens=70 * 64, max_seqs=70)
+    got = run_batches(session, requests, [list(range(70))], tail=8)
+    for r in (0, 1, 17, 63, 64, 65, 69):
+        ref = plain.forward(w, cfg, requests[r])
+        cut = max(1, len(requests[r]) - 8)
+        assert_close(dtype, got[r], ref[cut - 1:], f"{dtype} request {r} of a batch of 70")
+    assert session.cache.slots.n_free == 70
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_and_first_tokens(models, oracle, dtype):
     """A prompt of one token, then 230 tokens one by one across three page boundaries."""
     import edge_infer_amd as ei

@@ -555,11 +555,12 @@ def test_sample_refuses_bad_policies(lib):
 
 
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64, 65, 130, 256])
 @pytest.mark.parametrize("N,K", [(381, 96), (200, 200), (96, 256), (4096, 1024), (1000, 1384)])
 def test_gemm_bf16_skinny(lib, M, N, K):
     """The weight-streaming product for few rows: every slice count it may choose, widths
-    that are no multiple of the tile, and the same row alone or among others."""
+    that are no multiple of the tile, the same row alone or among others, and more than 64
+    rows (several blocks of 64 rows share each group of weight rows)."""
     torch.manual_seed(M * 7 + N)
     x = torch.randn(M, K, device=DEV).to(torch.bfloat16)
     w = torch.randn(N, K, device=DEV).to(torch.bfloat16)
@@ -595,7 +596,7 @@ def test_gemm_bf16_skinny(lib, M, N, K):
 
 @pytest.mark.parametrize("packed", [True, False])
 @pytest.mark.parametrize("M,I,K", [(1, 48, 256), (8, 1024, 512), (16, 16, 96), (33, 2048, 256),
-                                   (64, 208, 1000)])
+                                   (64, 208, 1000), (100, 2192, 256), (256, 48, 520)])
 def test_gemm_bf16_skinny_gated(lib, M, I, K, packed):
     """silu(x . gate) * (x . up) written by the few-rows kernel itself, from a weight whose
     rows alternate between 16 gate rows and their 16 up rows (all of K in one slice, also
@@ -630,9 +631,9 @@ def test_gemm_bf16_skinny_refuses_what_it_cannot_run(lib):
     with pytest.raises(KernelError, match="multiple of 8"):
         lib.gemm_bf16_skinny(x, w, torch.empty(1, 2, 32, device=DEV))
     w = torch.zeros(32, 96, device=DEV, dtype=torch.bfloat16)
-    x = torch.zeros(65, 96, device=DEV, dtype=torch.bfloat16)
-    with pytest.raises(KernelError, match="1..64"):
-        lib.gemm_bf16_skinny(x, w, torch.empty(1, 65, 32, device=DEV))
+    x = torch.zeros(257, 96, device=DEV, dtype=torch.bfloat16)
+    with pytest.raises(KernelError, match="1..256"):
+        lib.gemm_bf16_skinny(x, w, torch.empty(1, 257, 32, device=DEV))
     with pytest.raises(KernelError, match="do not agree"):       # packed for another n
         lib.gemm_bf16_skinny_packed(x[:2], lib.pack_weight(w), 48, torch.empty(1, 2, 48, device=DEV))
 
