@@ -1,15 +1,18 @@
 // Weight-streaming matrix product for few rows (decode): out[s][m][n] = partial sums of
-// X[m, :] . W[n, :] over the s-th slice of K, for M <= 64 rows of X.
+// X[m, :] . W[n, :] over the s-th slice of K, for M <= 256 rows of X.
 //
 // W is a bfloat16 checkpoint matrix [N, K] and is read exactly once, straight from global
 // memory into MFMA operand registers (v_mfma_f32_16x16x32_bf16: lane (row r, quarter c) holds
 // 8 consecutive k of row r).  It is read either in its stored layout or, faster, from a copy
-// packed at load time into whole MFMA tiles (see ei_gemm_bf16_skinny_packed).  X (tiny) is
-// staged through LDS one K-tile at a time.  A workgroup is 4, 6 or 8 waves, each owning 16
-// rows of W; K may be split over blockIdx.y, in which case every slice writes float32 partial
-// sums [slice, M, N] that the consuming kernel adds in slice order while it reads them
-// (deterministic, no atomics, and no device-wide fence: the kernel boundary orders the
-// writes before the reads).  The host picks the waves and slices per shape.
+// packed at load time into whole MFMA tiles (see ei_gemm_bf16_skinny_packed).  X (small) is
+// staged in LDS one K-tile at a time: with packed W it travels from global memory straight
+// into LDS (global_load_lds, no registers), otherwise through registers.  A workgroup is 4, 6
+// or 8 waves, each owning 16 rows of W, and takes 16, 32, 64 or 128 rows of X; more rows go to
+// further workgroups that share the weights through the L2 of their die.  K may be split over
+// blockIdx.y, in which case every slice writes float32 partial sums [slice, M, N] that the
+// consuming kernel adds in slice order while it reads them (deterministic, no atomics, and no
+// device-wide fence: the kernel boundary orders the writes before the reads).  The host picks
+// the waves and slices per shape.
 //
 // Accumulation is float32 throughout, as in the reference's cublasGemmEx call
 // (operators/src/cuda/execution.cu:319-323); the sums stay float32 and the consumer rounds
@@ -32,13 +35,13 @@ __device__ __forceinline__ const bf16_t* packed_piece(const bf16_t* Wp, int n_st
   return Wp + (static_cast<size_t>(kt) * n_strips + strip) * kPackedTile + lane * 8;
 }
 
-// Up to 64 rows of X, any K range.  A workgroup is WAVES waves, each owning 16 rows of W; X
-// travels through LDS one K-tile (256) at a time, two tiles of it alternate so that a tile
-// costs one barrier.  W has two register sets that are refilled piece by piece: as soon as
-// the products of one 32-wide step have read their piece, the same piece of the tile after
-// next is requested, so two tiles of W per wave are always on their way.  The loads of the
-// steady loop are unconditional (clamped addresses, zeros selected afterwards), so the number
-// outstanding is the same on every path and each wait leaves the younger loads in flight.
+// MB * 16 rows of X per workgroup, any K range.  A workgroup is WAVES waves, each owning 16
+// rows of W; X travels through LDS one K-tile (256) at a time, two tiles of it alternate so
+// that a tile costs one barrier.  W has two register sets that are refilled piece by piece:
+// as soon as the products of one 32-wide step have read their piece, the same piece of the
+// tile after next is requested, so two tiles of W per wave are always on their way.  The
+// loads of the steady loop are unconditional (clamped addresses), so the number outstanding
+// is the same on every path and each wait leaves the younger loads in flight.
 // Few K slices: for many rows the float32 partial sums (rows x N x 4 bytes a slice, written
 // in 64-byte pieces and read again by the consumer) cost more than the weights they save.
 //
@@ -114,31 +117,49 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   };
   // Rows past the last one repeat it (their sums are never stored), so every load is in
   // bounds and none is conditional; k past the end of the slice can only occur in its last
-  // tile, where the address is clamped and zeros are stored instead.
-  const int x_half = lane >> 5, x_chunk = lane & 31;
+  // tile, where the address is clamped (and, on the register path, zeros are stored).
+  // Row r keeps its 16-byte chunk g at place g ^ (r % 16), so that the operand reads (16
+  // rows, quarters c and c + 1 of a 32-wide step in one access group) touch every bank once.
+  const int x_half = lane >> 5, x_place = lane & 31;
   unsigned x_row[XLOADS];
+  int x_k[XLOADS];
 #pragma unroll
-  for (int i = 0; i < XLOADS; ++i)
-    x_row[i] = static_cast<unsigned>(min(2 * (wave + i * WAVES) + x_half, rows_here - 1)) * K;
+  for (int i = 0; i < XLOADS; ++i) {
+    const int row = 2 * min(wave + i * WAVES, PAIRS - 1) + x_half;   // surplus loads repeat the last pair
+    x_row[i] = static_cast<unsigned>(min(row, rows_here - 1)) * K;
+    x_k[i] = (x_place ^ (row & 15)) * 8;
+  }
+  // packed W (zeros past K, so whatever finite X meets them counts nothing): X goes from
+  // global memory straight into LDS, a wave load lands as one kilobyte at the pair's place
+  auto dma_x = [&](int buf, int tile) {
+    const int kb = k_begin + tile * KT;
+#pragma unroll
+    for (int i = 0; i < XLOADS; ++i) {
+      const int pair = min(wave + i * WAVES, PAIRS - 1);
+      const unsigned k = min(kb + x_k[i], k_end - 8);
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)(X + (x_row[i] + k)),
+          (__attribute__((address_space(3))) void*)(&xs[buf][pair * 2 * XS]), 16, 0, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);     // the waits below count the loads issued after these
+  };
+  // stored layout: through registers
   auto load_x = [&](int tile) {
     const int kb = k_begin + tile * KT;
-    const unsigned k = min(kb + x_chunk * 8, k_end - 8);
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i)
-      x_regs[i] = *reinterpret_cast<const u32x4*>(X + (x_row[i] + k));
+      x_regs[i] = *reinterpret_cast<const u32x4*>(X + (x_row[i] + min(kb + x_k[i], k_end - 8)));
   };
   // `last_tag`: the tile may be the last of the slice (k is checked)
   auto store_x = [&](int buf, int tile, auto last_tag) {
     constexpr bool check_k = decltype(last_tag)::value;
-    const bool k_ok = !check_k || k_begin + tile * KT + x_chunk * 8 < k_end;
+    const int kb = k_begin + tile * KT;
 #pragma unroll
     for (int i = 0; i < XLOADS; ++i) {
       const int pair = wave + i * WAVES;               // the same for the whole wave
-      const int row = 2 * pair + x_half;
-      // swizzled so that the operand reads below (16 rows, quarters c and c + 1 of a
-      // 32-wide step in one access group) touch every bank once
+      const bool k_ok = !check_k || kb + x_k[i] < k_end;
       if (PAIRS % WAVES == 0 || pair < PAIRS)
-        *reinterpret_cast<u32x4*>(&xs[buf][row * XS + (x_chunk ^ (row & 15)) * 8]) =
+        *reinterpret_cast<u32x4*>(&xs[buf][(2 * pair + x_half) * XS + x_place * 8]) =
             k_ok ? x_regs[i] : zero4;
     }
   };
@@ -154,25 +175,31 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
     const bf16_t* x_step[4];
 #pragma unroll
     for (int jj = 0; jj < 4; ++jj) x_step[jj] = x_base + (jj ^ (r16 >> 2)) * 32;
-    bf16x8 xf[2][MB];
+    // a unit: one 32-wide step of W against HB row tiles of X (128 rows take two units a
+    // step); the operands of the next unit are read while this one multiplies
+    constexpr int HB = MB < 4 ? MB : 4, UNITS = MB / HB;
+    bf16x8 xf[2][HB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
+    for (int mb = 0; mb < HB; ++mb)
       xf[0][mb] = *reinterpret_cast<const bf16x8*>(x_step[0] + mb * 16 * XS);
 #pragma unroll
-    for (int j = 0; j < JN; ++j) {
-      if (j + 1 < JN) {
+    for (int u = 0; u < JN * UNITS; ++u) {
+      const int j = u / UNITS, h = u % UNITS;
+      if (u + 1 < JN * UNITS) {
+        const int jn = (u + 1) / UNITS, hn = (u + 1) % UNITS;
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          xf[(j + 1) & 1][mb] = *reinterpret_cast<const bf16x8*>(
-              x_step[(j + 1) & 3] + mb * 16 * XS + ((j + 1) & 4) * 32);
+        for (int mb = 0; mb < HB; ++mb)
+          xf[(u + 1) & 1][mb] = *reinterpret_cast<const bf16x8*>(
+              x_step[jn & 3] + (hn * HB + mb) * 16 * XS + (jn & 4) * 32);
       }
-      // keep this order (reads of the next step, products, refill): left alone the
+      // keep this order (reads of the next unit, products, refill): left alone the
       // scheduler pairs every read with its use and gathers the refills at the end
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[set][j], xf[j & 1][mb], acc[mb], 0, 0, 0);
-      if (do_refill) load_w_piece(set, refill, j);
+      for (int mb = 0; mb < HB; ++mb)
+        acc[h * HB + mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[set][j], xf[u & 1][mb],
+                                                                   acc[h * HB + mb], 0, 0, 0);
+      if (do_refill && h == UNITS - 1) load_w_piece(set, refill, j);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -181,46 +208,97 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
   using Refill = std::true_type;
   using Last = std::false_type;
 
-  load_x(0);
-#pragma unroll
-  for (int j = 0; j < JN; ++j) load_w_piece(0, 0, j);
   using Inner = std::false_type;
   using MaybeLast = std::true_type;
-  if (n_iter == 1) {
-    store_x(0, 0, MaybeLast{});
-    __syncthreads();
-    compute(Set0{}, Last{}, 0);
-  } else {
+  if constexpr (PACKED) {
+    // s_waitcnt vmcnt(n): everything but the n youngest loads has arrived, i.e. the X tile
+    // requested before the n pieces of W that were requested after it.  A wave waits for
+    // its own part of the tile, the barrier then covers everybody's.  (No fence here: it
+    // would wait for the pieces of W as well.)
+    auto x_arrived = [&](auto younger_tag) {
+      constexpr int younger = decltype(younger_tag)::value;
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | (younger & 15) | ((younger >> 4) << 14));
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    using OneSet = std::integral_constant<int, JN>;
+    using TwoSets = std::integral_constant<int, 2 * JN>;
+    using None = std::integral_constant<int, 0>;
+    dma_x(0, 0);
 #pragma unroll
-    for (int j = 0; j < JN; ++j) load_w_piece(1, 1, j);
-    store_x(0, 0, Inner{});
-    load_x(1);
-    __syncthreads();
-    int i = 0;                            // even: tile i is in set 0
-    for (; i + 3 < n_iter; i += 2) {      // tiles i + 2 and i + 3 exist
-      compute(Set0{}, Refill{}, i + 2);
-      store_x(1, i + 1, Inner{});
-      load_x(i + 2);
-      __syncthreads();
-      compute(Set1{}, Refill{}, i + 3);
-      store_x(0, i + 2, Inner{});
-      load_x(i + 3);
-      __syncthreads();
+    for (int j = 0; j < JN; ++j) load_w_piece(0, 0, j);
+    if (n_iter == 1) {
+      x_arrived(OneSet{});
+      compute(Set0{}, Last{}, 0);
+    } else {
+#pragma unroll
+      for (int j = 0; j < JN; ++j) load_w_piece(1, 1, j);
+      x_arrived(TwoSets{});
+      int i = 0;                            // even: tile i is in set 0 and in X buffer 0
+      for (; i + 3 < n_iter; i += 2) {      // tiles i + 2 and i + 3 exist
+        dma_x(1, i + 1);
+        compute(Set0{}, Refill{}, i + 2);
+        x_arrived(OneSet{});
+        dma_x(0, i + 2);
+        compute(Set1{}, Refill{}, i + 3);
+        x_arrived(OneSet{});
+      }
+      if (i + 2 < n_iter) {                 // three tiles remain
+        dma_x(1, i + 1);
+        compute(Set0{}, Refill{}, i + 2);
+        x_arrived(OneSet{});
+        dma_x(0, i + 2);
+        compute(Set1{}, Last{}, 0);
+        x_arrived(None{});
+        compute(Set0{}, Last{}, 0);
+      } else {                              // two
+        dma_x(1, i + 1);
+        compute(Set0{}, Last{}, 0);
+        x_arrived(None{});
+        compute(Set1{}, Last{}, 0);
+      }
     }
-    if (i + 2 < n_iter) {                 // three tiles remain
-      compute(Set0{}, Refill{}, i + 2);
-      store_x(1, i + 1, Inner{});
-      load_x(i + 2);
-      __syncthreads();
-      compute(Set1{}, Last{}, 0);
-      store_x(0, i + 2, MaybeLast{});
+  } else {
+    load_x(0);
+#pragma unroll
+    for (int j = 0; j < JN; ++j) load_w_piece(0, 0, j);
+    if (n_iter == 1) {
+      store_x(0, 0, MaybeLast{});
       __syncthreads();
       compute(Set0{}, Last{}, 0);
-    } else {                              // two
-      compute(Set0{}, Last{}, 0);
-      store_x(1, i + 1, MaybeLast{});
+    } else {
+#pragma unroll
+      for (int j = 0; j < JN; ++j) load_w_piece(1, 1, j);
+      store_x(0, 0, Inner{});
+      load_x(1);
       __syncthreads();
-      compute(Set1{}, Last{}, 0);
+      int i = 0;                            // even: tile i is in set 0
+      for (; i + 3 < n_iter; i += 2) {      // tiles i + 2 and i + 3 exist
+        compute(Set0{}, Refill{}, i + 2);
+        store_x(1, i + 1, Inner{});
+        load_x(i + 2);
+        __syncthreads();
+        compute(Set1{}, Refill{}, i + 3);
+        store_x(0, i + 2, Inner{});
+        load_x(i + 3);
+        __syncthreads();
+      }
+      if (i + 2 < n_iter) {                 // three tiles remain
+        compute(Set0{}, Refill{}, i + 2);
+        store_x(1, i + 1, Inner{});
+        load_x(i + 2);
+        __syncthreads();
+        compute(Set1{}, Last{}, 0);
+        store_x(0, i + 2, MaybeLast{});
+        __syncthreads();
+        compute(Set0{}, Last{}, 0);
+      } else {                              // two
+        compute(Set0{}, Last{}, 0);
+        store_x(1, i + 1, MaybeLast{});
+        __syncthreads();
+        compute(Set1{}, Last{}, 0);
+      }
     }
   }
 
@@ -328,7 +406,7 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int max_splits) {
     if (!valid_slice_count(k_tiles, splits)) continue;
     const double tiles = static_cast<double>((k_tiles + splits - 1) / splits);
     double cost = 0.0;                                   // in strip-tiles (8 KB of W) per unit
-    tile_kernel_waves(n_strips, splits, (M + kGroupRows - 1) / kGroupRows, tiles, &cost);
+    tile_kernel_waves(n_strips, splits, (M + 2 * kGroupRows - 1) / (2 * kGroupRows), tiles, &cost);
     cost += 2.5 * splits * static_cast<double>(M) * N * 4.0 / kComputeUnits / 8192.0;
     if (cost < best_cost - 1e-9) {
       best_cost = cost;
@@ -376,7 +454,7 @@ int launch_skinny(const void* X, const void* W, float* out, void* gated_out, int
     EI_REQUIRE(splits == 1, "gemm_bf16_skinny_gated: K cannot be sliced");
     EI_REQUIRE(N % 32 == 0, "gemm_bf16_skinny_gated: N must be a multiple of 32 (gate and up strips)");
   }
-  const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const int MB = M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 || !PACKED ? 4 : 8));
   const int k_tiles = (K + kTile - 1) / kTile;
   EI_REQUIRE(splits >= 1 && splits <= k_tiles, "gemm_bf16_skinny: bad slice count");
   EI_REQUIRE(valid_slice_count(k_tiles, splits), "gemm_bf16_skinny: slice count leaves an empty slice");
@@ -388,8 +466,11 @@ int launch_skinny(const void* X, const void* W, float* out, void* gated_out, int
     launch_tile_kernel<1, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
   } else if (MB == 2) {
     launch_tile_kernel<2, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
-  } else {
+  } else if (MB == 4) {
     launch_tile_kernel<4, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
+  } else {
+    if constexpr (PACKED)
+      launch_tile_kernel<8, PACKED, GATED>(w, x, out, g, M, N, K, k_per_split, splits, stream);
   }
   EI_LAUNCH_CHECK();
 }

@@ -418,7 +418,7 @@ def skinny_gemm_splits(rows: int, n: int, k: int) -> int:
 
 
 # most rows for which the weight-streaming product is taken instead of the library's
-SKINNY_ROWS = int(os.environ.get("EDGE_INFER_SKINNY_ROWS", "128"))
+SKINNY_ROWS = int(os.environ.get("EDGE_INFER_SKINNY_ROWS", "256"))
 if not 1 <= SKINNY_ROWS <= 256:
     raise KernelError("EDGE_INFER_SKINNY_ROWS must lie in 1..256")
 
