@@ -299,7 +299,8 @@ def test_one_layer_of_the_8b_shape(tmp_path, dtype):
     """Layer sizes of Qwen3-8B (hidden 4096, 32 heads, 8 kv heads, head_dim 128,
     intermediate 12288) with one layer and a small vocabulary: the kernels that the big
     model uses (matrix-core attention, few-rows and library products at K = 4096 and
-    12288) against the plain implementation, whole and token by token, two sequences."""
+    12288) against the plain implementation, whole and token by token, two sequences.  The
+    370 prompt rows of the first step are beyond the few-rows product and go to the library."""
     import edge_infer_amd as ei
     cfg = ei.Qwen3Config(vocab_size=1000, hidden_size=4096, num_hidden_layers=1,
                          num_attention_heads=32, num_key_value_heads=8, head_dim=128,
@@ -308,23 +309,23 @@ def test_one_layer_of_the_8b_shape(tmp_path, dtype):
                          tie_word_embeddings=False)
     folder = ei.write_model_folder(tmp_path / "layer8b", cfg, seed=2)
     pcfg, pw = plain.read_folder(folder)
-    a, b = random_ids(1000, 150, 5), random_ids(1000, 70, 6)
+    a, b = random_ids(1000, 330, 5), random_ids(1000, 70, 6)
     ref_a, ref_b = plain.forward(pw, pcfg, a), plain.forward(pw, pcfg, b)
     model = ei.load_model(folder, dtype=dtype)
-    session = ei.Session(model, max_tokens=512, max_seqs=2)
+    session = ei.Session(model, max_tokens=1024, max_seqs=2)
     sa, sb = session.begin(), session.begin()
-    logits = session.step([(sa, a[:130], list(range(130))), (sb, b[:60], list(range(60)))])
-    assert_close(dtype, logits[:130], ref_a[:130], f"8B-shape layer {dtype} prefill a")
-    assert_close(dtype, logits[130:], ref_b[:60], f"8B-shape layer {dtype} prefill b")
+    logits = session.step([(sa, a[:310], list(range(310))), (sb, b[:60], list(range(60)))])
+    assert_close(dtype, logits[:310], ref_a[:310], f"8B-shape layer {dtype} prefill a")
+    assert_close(dtype, logits[310:], ref_b[:60], f"8B-shape layer {dtype} prefill b")
     rows_a, rows_b = [], []
     for t in range(20):
-        entries = [(sa, [a[130 + t]], [0])]
+        entries = [(sa, [a[310 + t]], [0])]
         if t < 10:
             entries.append((sb, [b[60 + t]], [0]))
         out = session.step(entries)
         rows_a.append(out[0])
         if t < 10:
             rows_b.append(out[1])
-    assert_close(dtype, torch.stack(rows_a), ref_a[130:], f"8B-shape layer {dtype} decode a")
+    assert_close(dtype, torch.stack(rows_a), ref_a[310:], f"8B-shape layer {dtype} decode a")
     assert_close(dtype, torch.stack(rows_b), ref_b[60:], f"8B-shape layer {dtype} decode b")
     assert session.graph_replays > 0
