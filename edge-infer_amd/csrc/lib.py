@@ -70,7 +70,8 @@ _SIGNATURES = {
         "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
         "ei_argmax_partial_size": [c_int, c_int],
         "ei_sample": [c_void_p, c_int, c_int, c_float, c_float, c_int, c_ulonglong, c_void_p,
-                      c_void_p, c_void_p, c_void_p, c_void_p],
+                      c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
+        "ei_sample_scratch_size": [c_int, c_int],
     },
 }
 
@@ -388,8 +389,15 @@ def argmax(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None, parti
     _check(lib, status, "argmax")
 
 
+def sample_scratch_size(rows: int, vocab: int) -> int:
+    """int32 elements of zeroed scratch that `sample` takes for many blocks a row (0: none)."""
+    return library("sampling").ei_sample_scratch_size(rows, vocab)
+
+
 def sample(logits, temperature, top_p, top_k, seed, streams, counters, tokens,
-           probabilities=None) -> None:
+           probabilities=None, scratch=None) -> None:
+    """`scratch` (int32, zero before its first use, see `sample_scratch_size`) lets a wide
+    vocabulary be searched by many blocks a row; the tokens are the same without it."""
     lib = library("sampling")
     rows, vocab = logits.shape
     if tokens.numel() < rows or streams.numel() < rows or counters.numel() < rows:
@@ -400,7 +408,9 @@ def sample(logits, temperature, top_p, top_k, seed, streams, counters, tokens,
                            _gpu(counters, "counters", torch.int32),
                            _gpu(tokens, "tokens", torch.int32),
                            None if probabilities is None
-                           else _gpu(probabilities, "probabilities", torch.float32), _stream())
+                           else _gpu(probabilities, "probabilities", torch.float32),
+                           None if scratch is None else _gpu(scratch, "scratch", torch.int32),
+                           0 if scratch is None else scratch.numel(), _stream())
     _check(lib, status, "sample")
 
 

@@ -20,6 +20,7 @@ class Sampler:
         self._probabilities = torch.empty(1024, dtype=torch.float32, device=self.device)
         self._meta = torch.empty(2048, dtype=torch.int32, device=self.device)
         self._partial = None          # scratch of the greedy search over a wide vocabulary
+        self._scratch = None          # zeroed scratch of sampling from a wide vocabulary
         self._last_rows = 0
 
     def _reserve(self, rows: int) -> None:
@@ -46,8 +47,12 @@ class Sampler:
                 raise ValueError("one stream number and one counter per row are needed")
             host = torch.tensor(list(streams) + list(counters), dtype=torch.int32)
             self._meta[:2 * rows].copy_(host)
+            need = lib.sample_scratch_size(rows, vocab)
+            if need and (self._scratch is None or self._scratch.numel() < need):
+                self._scratch = torch.zeros(need, dtype=torch.int32, device=self.device)
             lib.sample(logits, params.temperature, params.top_p, params.top_k, params.seed,
-                       self._meta[:rows], self._meta[rows:2 * rows], tokens, probabilities)
+                       self._meta[:rows], self._meta[rows:2 * rows], tokens, probabilities,
+                       self._scratch if need else None)
         return tokens
 
     def __call__(self, logits, params, streams, counters) -> List[int]:

@@ -524,24 +524,48 @@ def test_sample_reference_distribution(lib):
 
 
 def test_sample_large_vocabulary_matches_plain(lib):
+    """Without scratch (one block a row) and with it (many blocks a row gather the pairs that
+    can belong to the top k): the same tokens as the plain sampler, also where the gathered
+    list overflows (thousands of ties, everything equal) or is tied beyond 1024 pairs, and
+    in later calls with other row counts on the same scratch."""
     V = 151936
     g = torch.Generator().manual_seed(3)
-    logits = (torch.randn(6, V, generator=g) * 2.5)
+    logits = (torch.randn(7, V, generator=g) * 2.5)
     logits[2, :5000] = 6.0                         # thousands of ties around the threshold
     logits[3, 100:104] = 30.0                      # ties at the very top
     logits[4, :] = -1.0                            # everything equal
     logits[5, 17] = float("nan")
+    logits[6, 1000:3000] = 9.5                     # 2000 ties: they fit the list, not the tie table
     dev = logits.to(DEV)
-    streams = torch.tensor([0, 1, 2, 3, 4, 5], dtype=torch.int32, device=DEV)
-    counters = torch.tensor([0, 5, 9, 1, 2, 3], dtype=torch.int32, device=DEV)
+    streams = torch.tensor([0, 1, 2, 3, 4, 5, 6], dtype=torch.int32, device=DEV)
+    counters = torch.tensor([0, 5, 9, 1, 2, 3, 4], dtype=torch.int32, device=DEV)
+    need = lib.sample_scratch_size(7, V)
+    assert need > 0 and lib.sample_scratch_size(7, 5000) == 0
+    scratch = torch.zeros(need, dtype=torch.int32, device=DEV)
     for temperature, top_p, top_k in [(0.8, 0.95, 50), (1.3, 1.0, 1024), (0.7, 0.5, 20),
                                       (1.0, 1.0, 3)]:
-        tokens = torch.empty(6, dtype=torch.int32, device=DEV)
+        tokens = torch.empty(7, dtype=torch.int32, device=DEV)
         lib.sample(dev, temperature, top_p, top_k, 42, streams, counters, tokens)
-        for r in range(6):
+        wide = torch.empty(7, dtype=torch.int32, device=DEV)
+        prob = torch.empty(7, device=DEV)
+        lib.sample(dev, temperature, top_p, top_k, 42, streams, counters, wide, prob, scratch)
+        for r in range(7):
             u = plain.uniform(42, int(streams[r]), int(counters[r]))
-            assert tokens[r].item() == plain.sample(logits[r].numpy(), temperature, top_p, top_k, u), \
-                (r, temperature, top_p, top_k)
+            expected = plain.sample(logits[r].numpy(), temperature, top_p, top_k, u)
+            assert tokens[r].item() == expected, (r, temperature, top_p, top_k)
+            assert wide[r].item() == expected, ("many blocks", r, temperature, top_p, top_k)
+        # fewer rows on the same scratch, from the second row on
+        part = torch.empty(3, dtype=torch.int32, device=DEV)
+        lib.sample(dev[1:4], temperature, top_p, top_k, 42, streams[1:4], counters[1:4], part,
+                   None, scratch)
+        assert part.tolist() == wide[1:4].tolist()
+    # every call left what must start at zero at zero (bins and counts; lists may hold anything)
+    per_row = need // 7
+    view = scratch.view(7, per_row)
+    assert int(view[:, :4096 + 4].abs().sum().item()) == 0
+    from edge_infer_amd.csrc.lib import KernelError
+    with pytest.raises(KernelError, match="too small"):
+        lib.sample(dev, 1.0, 1.0, 5, 42, streams, counters, tokens, None, scratch[:100])
 
 
 def test_sample_refuses_bad_policies(lib):
