@@ -19,6 +19,10 @@ class Sampler:
         self._tokens = torch.empty(1024, dtype=torch.int32, device=self.device)
         self._probabilities = torch.empty(1024, dtype=torch.float32, device=self.device)
         self._meta = torch.empty(2048, dtype=torch.int32, device=self.device)
+        # stream numbers and counters travel through pinned memory; two buffers in turn, so
+        # that filling one does not disturb a copy of the other that is still queued
+        self._meta_host = [torch.empty(2048, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self._meta_turn = 0
         self._partial = None          # scratch of the greedy search over a wide vocabulary
         self._scratch = None          # zeroed scratch of sampling from a wide vocabulary
         self._last_rows = 0
@@ -28,6 +32,8 @@ class Sampler:
             self._tokens = torch.empty(rows, dtype=torch.int32, device=self.device)
             self._probabilities = torch.empty(rows, dtype=torch.float32, device=self.device)
             self._meta = torch.empty(2 * rows, dtype=torch.int32, device=self.device)
+            self._meta_host = [torch.empty(2 * rows, dtype=torch.int32, pin_memory=True)
+                               for _ in range(2)]
 
     def sample_device(self, logits: torch.Tensor, params: SamplingParams, streams: Sequence[int],
                       counters: Sequence[int]) -> torch.Tensor:
@@ -45,8 +51,10 @@ class Sampler:
         else:
             if len(streams) != rows or len(counters) != rows:
                 raise ValueError("one stream number and one counter per row are needed")
-            host = torch.tensor(list(streams) + list(counters), dtype=torch.int32)
-            self._meta[:2 * rows].copy_(host)
+            host = self._meta_host[self._meta_turn]
+            self._meta_turn ^= 1
+            host[:2 * rows] = torch.tensor(list(streams) + list(counters), dtype=torch.int32)
+            self._meta[:2 * rows].copy_(host[:2 * rows], non_blocking=True)
             need = lib.sample_scratch_size(rows, vocab)
             if need and (self._scratch is None or self._scratch.numel() < need):
                 self._scratch = torch.zeros(need, dtype=torch.int32, device=self.device)
