@@ -567,8 +567,8 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
                    const int32_t* page_table, int table_width, bf16_t* out, float* part_o,
                    float* part_ml, int nq, int nkv, int head_blocks, int window, float scale,
                    int n_splits, int waves) {
-  if constexpr (GB <= 4) {               // larger head blocks: the merge buffers of 16 waves
-    if (waves == 16) {                   // would not fit in LDS
+  if constexpr (GB <= 4) {               // the caller gives 16 waves at most 4 heads a block
+    if (waves == 16) {
       attn_decode_kernel<D, GB, 16><<<grid, 16 * EI_WAVE, 0, stream>>>(
           q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
           head_blocks, window, scale, n_splits);
@@ -666,7 +666,10 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
   EI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention_decode: split scratch missing");
   EI_REQUIRE(window >= 0, "attention_decode: negative window");
   const int G = nq / nkv;
-  const int GB = G >= 8 ? (G >= 16 ? 16 : 8) : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
+  // heads of a kv group that one block takes; blocks of 16 waves take at most 4 (their merge
+  // buffers grow with both), a larger group then has several blocks per kv head
+  int GB = G >= 8 ? (G >= 16 ? 16 : 8) : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
+  if (waves == 16 && GB > 4) GB = 4;
   const int head_blocks = (G + GB - 1) / GB;
   EI_REQUIRE(static_cast<long long>(nkv) * head_blocks <= 65535, "attention_decode: too many heads");
   dim3 grid(rows, nkv * head_blocks, n_splits);

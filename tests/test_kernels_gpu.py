@@ -390,7 +390,7 @@ def test_attention_window_edge(lib, dtype, window):
             close(out, expected, dtype)
 
 
-@pytest.mark.parametrize("nq,nkv,D,splits", [(32, 8, 128, 1), (32, 8, 128, 4), (8, 8, 64, 3),
+@pytest.mark.parametrize("nq,nkv,D,splits", [(32, 8, 128, 1), (32, 8, 128, 4), (8, 8, 64, 3), (64, 8, 128, 1),
                                              (6, 2, 128, 2), (20, 1, 64, 5), (16, 1, 128, 32),
                                              (2, 1, 64, 1)])
 @pytest.mark.parametrize("waves", [4, 16])
