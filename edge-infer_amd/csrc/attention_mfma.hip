@@ -37,7 +37,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
                    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table,
                    int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
                    float* __restrict__ part_ml, int nq, int nkv, int head_blocks, int window,
-                   float scale, int n_splits) {
+                   float scale, int n_splits, const int32_t* __restrict__ longest) {
   constexpr int DJ = D / 32;            // MFMA steps over the head dimension
   constexpr int LPR = D / 8;            // lanes that cover one value row with 16-byte loads
   constexpr int KPI = EI_WAVE / LPR;    // value rows per load instruction
@@ -76,9 +76,21 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   // slices are cut at page boundaries so that they do not depend on the tile size
   const int lo_page = lo_key / EI_PAGE, hi_page = pos / EI_PAGE;
   const int pages = hi_page - lo_page + 1;
-  const int per = (pages + n_splits - 1) / n_splits;
+  // A slice is the same number of pages for every sequence of the step: the longest one's
+  // share (`longest`: the most tokens any sequence holds, read on the device so that a captured
+  // step follows it).  Sequences of unequal lengths then give blocks of about equal work, and
+  // the later slices of a short sequence are empty.  Without it (or with a window, where the
+  // ranges start at different pages) every sequence is cut into n_splits equal parts.
+  int per = (pages + n_splits - 1) / n_splits;
+  if (longest != nullptr && window <= 0) {
+    const int most_pages = (*longest + EI_PAGE - 1) / EI_PAGE;
+    per = max(1, (most_pages + n_splits - 1) / n_splits);
+  }
   const int tile_begin = max(first_tile, (lo_page + split * per) * (EI_PAGE / kTile));
-  const int tile_end = min(last_tile + 1, (lo_page + (split + 1) * per) * (EI_PAGE / kTile));
+  // (the last slice takes whatever is left, so that no key is lost should `longest` be short)
+  const int tile_end = split == n_splits - 1
+                           ? last_tile + 1
+                           : min(last_tile + 1, (lo_page + (split + 1) * per) * (EI_PAGE / kTile));
   (void)total_tiles;
 
   float m_run = kLowest, l_run = 0.f;              // state of head r16 (same in all four c)
@@ -566,18 +578,18 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
                    const bf16_t* v, const int32_t* row_pos, const int32_t* row_seq,
                    const int32_t* page_table, int table_width, bf16_t* out, float* part_o,
                    float* part_ml, int nq, int nkv, int head_blocks, int window, float scale,
-                   int n_splits, int waves) {
+                   int n_splits, int waves, const int32_t* longest) {
   if constexpr (GB <= 4) {               // the caller gives 16 waves at most 4 heads a block
     if (waves == 16) {
       attn_decode_kernel<D, GB, 16><<<grid, 16 * EI_WAVE, 0, stream>>>(
           q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-          head_blocks, window, scale, n_splits);
+          head_blocks, window, scale, n_splits, longest);
       return;
     }
   }
   attn_decode_kernel<D, GB, 4><<<grid, 4 * EI_WAVE, 0, stream>>>(
         q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-        head_blocks, window, scale, n_splits);
+        head_blocks, window, scale, n_splits, longest);
 }
 
 }  // namespace
@@ -650,13 +662,14 @@ extern "C" int ei_attn_decode_mfma_supported(int D, int G) {
 
 // q, out: [rows, nq, D] bfloat16, one row per sequence (row_seq < 0: padding row);
 // pages: [n_pages, nkv, 64, D]; n_splits > 1 needs part_o [rows, nq, n_splits, D] and
-// part_ml [rows, nq, n_splits, 2] float32.
+// part_ml [rows, nq, n_splits, 2] float32.  longest (or null): one int32 on the device, the most
+// tokens that a sequence of this step holds; slices are then that sequence's share for all.
 extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, const void* v_pages,
                                         const int32_t* row_pos, const int32_t* row_seq,
                                         const int32_t* page_table, int table_width, void* out,
                                         float* part_o, float* part_ml, int rows, int nq, int nkv,
                                         int D, int window, float scale, int n_splits,
-                                        int waves, hipStream_t stream) {
+                                        int waves, const int32_t* longest, hipStream_t stream) {
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
   EI_REQUIRE(waves == 4 || waves == 16, "attention_decode: a block has 4 or 16 waves");
   EI_REQUIRE(D == 64 || D == 128, "attention_decode: this kernel takes head_dim 64 or 128");
@@ -680,7 +693,7 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
 #define EI_DECODE(DD, GG)                                                                     \
   launch_decode<DD, GG>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table, table_width,  \
                         oo, part_o, part_ml, nq, nkv, head_blocks, window, scale, n_splits,   \
-                        waves)
+                        waves, longest)
 #define EI_DECODE_G(DD)            \
   switch (GB) {                    \
     case 1: EI_DECODE(DD, 1); break;   \

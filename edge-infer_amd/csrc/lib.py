@@ -51,7 +51,7 @@ _SIGNATURES = {
                                       c_int, c_int, c_float, c_void_p],
         "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                     c_int, c_int, c_float, c_int, c_int, c_void_p],
+                                     c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
     },
     "gemm_f32": {
         "ei_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_longlong, c_longlong,
@@ -326,10 +326,12 @@ def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, 
 
 def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,
                           n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
-                          part_ml=None, waves=4) -> None:
+                          part_ml=None, waves=4, longest=None) -> None:
     """bfloat16 decode attention on the matrix cores: one query row per sequence.  `waves`
     (4 or 16) of a block share its key range tile by tile; 16 suit few sequences (few
-    blocks), whose ranges then need fewer slices or none."""
+    blocks), whose ranges then need fewer slices or none.  `longest` (int32 [1] on the
+    device): the most tokens a sequence of the step holds; every sequence's range is then
+    cut into slices of the longest one's share, so that unequal lengths give equal blocks."""
     lib = library("attention_mfma")
     n = q.shape[0]
     if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
@@ -352,7 +354,8 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
         page_table.shape[-1], _gpu(out, "out", torch.bfloat16),
         None if part_o is None else _gpu(part_o, "part_o", torch.float32),
         None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
-        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves), _stream())
+        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves),
+        None if longest is None else _gpu(longest, "longest", torch.int32), _stream())
     _check(lib, status, "attention_decode")
 
 

@@ -4,7 +4,7 @@ A step runs the tokens it is given as one packed batch of rows.  Only position
 encoding, cache store and attention read the metadata; every other operation is
 row-wise.  All of it lives in one int32 buffer:
 
-  tokens[N] row_pos[N] row_seq[N] want_rows[W]
+  longest[1] tokens[N] row_pos[N] row_seq[N] want_rows[W]
   per attention item size: item_seq[I] item_row0[I] item_npos[I]   (prefill)
   decode items: item_seq[B] item_row0[B] item_npos[B]             (decode)
   per key/value group: page_table[B, width]
@@ -108,7 +108,10 @@ class StepPlan:
         return seq, row0, npos
 
     def sections(self, page_tables: Sequence[np.ndarray]) -> List[Tuple[str, np.ndarray]]:
-        out = [("tokens", self.tokens), ("row_pos", self.row_pos), ("row_seq", self.row_seq),
+        # longest: the most tokens any sequence holds after this step (decode attention sizes
+        # its slices by it); first, so that its place never depends on the batch
+        out = [("longest", np.asarray([self.max_context], dtype=np.int32)),
+               ("tokens", self.tokens), ("row_pos", self.row_pos), ("row_seq", self.row_seq),
                ("want_rows", self.want_rows)]
         if self.decode:
             seq, row0, npos = self.decode_items()
@@ -164,6 +167,10 @@ class DeviceMeta:
         self.n_want = int(plan.want_rows.size)
 
     # views ------------------------------------------------------------
+    @property
+    def longest(self):
+        return self._views["longest"]
+
     @property
     def tokens(self):
         return self._views["tokens"]

@@ -102,7 +102,7 @@ class Attention:
                                           page_table, out, spec.n_heads, spec.n_kv_heads,
                                           spec.head_dim, window=spec.window, scale=self.scale,
                                           n_splits=splits, part_o=part_o, part_ml=part_ml,
-                                          waves=waves)
+                                          waves=waves, longest=meta.longest)
             else:
                 item_seq, item_row0, item_npos, n_items = meta.decode_items()
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,

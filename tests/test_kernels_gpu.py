@@ -282,7 +282,7 @@ def items_for(lib, starts, counts, group, per=None):
 
 
 def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
-                  boost=None, kernel="generic", waves=4):
+                  boost=None, kernel="generic", waves=4, longest=None):
     """Fill a paged cache with random keys and values, run the kernel for the last
     `counts[b]` positions of each sequence, return (kernel output, plain output)."""
     torch.manual_seed(seed)
@@ -321,7 +321,9 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     elif kernel == "decode_mfma":
         lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
                                   cache.table_dev, out, nq, nkv, D, window=window,
-                                  n_splits=splits, part_o=part_o, part_ml=part_ml, waves=waves)
+                                  n_splits=splits, part_o=part_o, part_ml=part_ml, waves=waves,
+                                  longest=None if longest is None else torch.tensor(
+                                      [longest], dtype=torch.int32, device=DEV))
     else:
         lib.attention(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0, item_npos,
                       n_items, pos, seq, cache.table_dev, out, nq, nkv, D, window=window,
@@ -402,6 +404,20 @@ def test_attention_decode_on_the_matrix_cores(lib, nq, nkv, D, splits, waves):
     out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, starts=starts,
                                   counts=[1] * len(starts), splits=splits, kernel="decode_mfma",
                                   waves=waves)
+    close(out, expected, torch.bfloat16)
+
+
+@pytest.mark.parametrize("splits,waves", [(2, 4), (5, 4), (32, 4), (3, 16)])
+@pytest.mark.parametrize("longest", ["exact", "short", "long"])
+def test_attention_decode_slices_of_the_longest_sequences_share(lib, splits, waves, longest):
+    """Slices sized by the longest sequence (a number on the device): sequences of very
+    unequal lengths, a stated length that is exact, too short (the last slice still takes
+    what is left) or longer than any sequence."""
+    starts = [0, 5, 63, 64, 200, 1029, 2300, 17]
+    stated = {"exact": 2301, "short": 700, "long": 4000}[longest]
+    out, expected = run_attention(lib, torch.bfloat16, 32, 8, 128, starts=starts,
+                                  counts=[1] * len(starts), splits=splits, kernel="decode_mfma",
+                                  waves=waves, longest=stated, seed=3)
     close(out, expected, torch.bfloat16)
 
 
