@@ -363,7 +363,7 @@ constexpr int kMaxRows = 256;
 // per unit all run at once, so the unit with the most blocks sets the time; many more blocks
 // than that even out.  Every block also costs a start (about 3 strip-tiles).  Near ties go
 // to the larger block, which shares a tile of X among more waves.  `row_groups` blocks work
-// on every strip group (more than 64 rows of X).
+// on every strip group (more rows of X than one block takes).
 int tile_kernel_waves(int n_strips, int splits, int row_groups, double tiles_per_slice,
                       double* cost_out) {
   int best = 8;
@@ -479,7 +479,8 @@ int launch_skinny(const void* X, const void* W, float* out, void* gated_out, int
 
 // X: [M, K] bfloat16, W: [N, K] bfloat16, out: [splits, M, N] float32 (slice s holds the
 // sums over the s-th part of K).  K must be a multiple of 8 (16-byte loads), M at most 256
-// (beyond 64 rows, blocks of 64 rows each share the weights through the L2 of their die).
+// (beyond 128 rows, or 64 in the stored layout, several blocks share the weights through the
+// L2 of their die).
 extern "C" int ei_gemm_bf16_skinny(const void* X, const void* W, float* out, int M, int N, int K,
                                    int splits, hipStream_t stream) {
   return launch_skinny<false, false>(X, W, out, nullptr, M, N, K, splits, stream);
