@@ -12,10 +12,15 @@ their caches.  Beyond the reference, a session can serve a batch of prompts
 (`new_session(max_batch=8)`, `session.generate_batch`) and exposes the step function
 (`session.step`).  Model types: "qwen3_bf16" (the reference's name) and
 "qwen3_fp32" for the true 32-bit path.
+
+The reference's procedural wrappers over one implicit session are here too
+(model_bridge.cpp:159-215,274-283): `init_model`, `generate_text_stream`,
+`set_default_device`, `get_default_device`, `is_cuda_available`.
 """
 from __future__ import annotations
 
 import json
+import sys
 from pathlib import Path
 from typing import Mapping, Optional
 
@@ -97,3 +102,69 @@ class Model:
 
 def is_gpu_available() -> bool:
     return torch.cuda.is_available()
+
+
+# -- the procedural interface: one implicit model and session ---------------------------
+_compat = {"model": None, "session": None, "busy": False}
+
+
+class _Operation:
+    """One call of the procedural interface at a time: a callback that calls back in is an
+    error, as in the reference (model_bridge.cpp:165-168)."""
+
+    def __enter__(self):
+        if _compat["busy"]:
+            raise RuntimeError("the runtime is busy with another operation")
+        _compat["busy"] = True
+
+    def __exit__(self, *exc):
+        _compat["busy"] = False
+        return False
+
+
+def init_model(config: Mapping, weights: Mapping[str, torch.Tensor],
+               model_type: str = "qwen3_bf16") -> bool:
+    """Replace the implicit model and its session (default capacity); on failure the
+    previous ones stay, the reason goes to stderr and False comes back."""
+    with _Operation():
+        try:
+            model = Model(config, weights, model_type)
+            session = model.new_session()
+        except Exception as error:                      # the reference catches everything here
+            print(f"Error initializing model: {error}", file=sys.stderr)
+            return False
+        _compat["model"], _compat["session"] = model, session
+        return True
+
+
+def generate_text_stream(input_ids, callback, max_length: int = 100, temperature: float = 1.0,
+                         top_p: float = 0.9, top_k: int = 50) -> None:
+    """`Session.generate` on the implicit session (note the other default of top_k)."""
+    with _Operation():
+        if _compat["session"] is None:
+            raise RuntimeError("Model not initialized")
+        _compat["session"].generate(list(input_ids), callback, max_length=max_length,
+                                    temperature=temperature, top_p=top_p, top_k=top_k)
+
+
+def set_default_device(device: str) -> bool:
+    """Only "cuda" can be the default here: there is no CPU path."""
+    with _Operation():
+        try:
+            if str(device) != "cuda" and not str(device).startswith("cuda:"):
+                raise ValueError(f"unsupported device '{device}': this library runs on the GPU only")
+            if not torch.cuda.is_available():
+                raise RuntimeError("cuda requested but no GPU is available")
+            return True
+        except Exception as error:
+            print(f"Error setting default device: {error}", file=sys.stderr)
+            return False
+
+
+def get_default_device() -> str:
+    return "cuda"
+
+
+def is_cuda_available() -> bool:
+    """The reference's name; `is_gpu_available` is the same."""
+    return is_gpu_available()

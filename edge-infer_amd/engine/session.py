@@ -117,6 +117,12 @@ class Session:
         return self.cache.max_seq_tokens
 
     @property
+    def speculative(self) -> bool:
+        """Always False (the reference's sessions say whether they draft with a second model,
+        bindings/python/model_bridge.cpp:256; this library has no such sessions)."""
+        return False
+
+    @property
     def max_batch(self) -> int:
         return self.cache.n_slots
 

@@ -270,6 +270,33 @@ def test_greedy_generation_through_the_entry_point(folders, oracle, name, dtype)
         assert cut == got[0][:got[0].index(stop)]
 
 
+def test_procedural_interface_generates_like_a_session(folders, oracle):
+    """init_model / generate_text_stream (bindings/python/model_bridge.cpp:171-193): the
+    implicit session gives the tokens of an explicit one; a failed init keeps the old model;
+    a callback that calls back in is refused."""
+    from edge_infer_amd import api
+    cfg, w = oracle["A"]
+    prompt = requests_for("A", [9], seed=77)[0]
+    config, weights, model_type = api.load_checkpoint(folders["A"], "qwen3_fp32")
+    assert api.init_model(config, weights, model_type) is True
+    got = []
+    api.generate_text_stream(prompt, got.append, max_length=len(prompt) + 6, top_k=1)
+    expected = plain.generate(w, cfg, prompt, max_length=len(prompt) + 6)
+    assert got == expected
+    assert api.init_model({"architectures": ["NoSuchModel"]}, {}, "qwen3_fp32") is False
+    again = []
+    api.generate_text_stream(prompt, again.append, max_length=len(prompt) + 6, top_k=1)
+    assert again == got
+
+    def nested(token):
+        with pytest.raises(RuntimeError, match="busy"):
+            api.generate_text_stream(prompt, lambda t: None, max_length=len(prompt) + 1)
+    api.generate_text_stream(prompt, nested, max_length=len(prompt) + 2, top_k=1)
+    session = api._compat["session"]
+    assert session.speculative is False and session.capacity == min(4096, cfg["max_position_embeddings"])
+    api._compat["model"] = api._compat["session"] = None
+
+
 def test_seeded_sampling_is_the_same_alone_and_in_a_batch(folders, oracle):
     """Configuration B's workload: temperature 0.8 with a seeded sampler.  Every drawn
     token equals the plain sampler's draw from the plain logits of the same prefix."""

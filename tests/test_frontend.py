@@ -86,3 +86,23 @@ def test_command_line_generates_from_ids_and_from_text(tmp_path):
     run = subprocess.run(base, input="hello\nquit\n", capture_output=True, text=True, timeout=300)
     assert run.returncode == 0, run.stderr[-2000:]
     assert "Assistant:" in run.stdout and "Chat started" in run.stdout
+
+
+def test_procedural_interface_without_a_model(capsys):
+    """bindings/python/model_bridge.cpp:159-215: generating before init_model is an error;
+    a failed init_model reports on stderr, returns False and leaves things as they were;
+    only the GPU can be the default device."""
+    from edge_infer_amd import api
+    assert api._compat["session"] is None
+    with pytest.raises(RuntimeError, match="Model not initialized"):
+        api.generate_text_stream([1, 2, 3], lambda token: None)
+    assert api.init_model({"architectures": ["NoSuchModel"]}, {}, "qwen3_bf16") is False
+    assert "Error initializing model" in capsys.readouterr().err
+    assert api.init_model({}, {}, "llama") is False          # a type this library does not have
+    assert api._compat["session"] is None and api._compat["busy"] is False
+    assert api.set_default_device("cpu") is False
+    assert "Error setting default device" in capsys.readouterr().err
+    assert api.get_default_device() == "cuda"
+    assert api.is_cuda_available() == api.is_gpu_available()
+    import inspect
+    assert inspect.signature(api.generate_text_stream).parameters["top_k"].default == 50
