@@ -9,6 +9,7 @@ session as it was; the reference holds the same contract, runtime/src/qwen3.cpp:
 """
 from __future__ import annotations
 
+import os
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -87,8 +88,11 @@ class Session:
         self._item_sizes = model.attention_item_sizes()
         self.steps_run = 0
         # decode steps are replayed from HIP graphs unless the model has an operation
-        # that is not safe to capture (see DecoderModel.capture_safe)
-        self.graphs = bool(graphs) and model.capture_safe()
+        # that is not safe to capture (see DecoderModel.capture_safe) or the caller or the
+        # environment says no: EDGE_INFER_ENABLE_QWEN3_GRAPH=0 (the reference's switch,
+        # runtime/src/qwen3.cpp:9-12, where graphs are off unless it is 1)
+        self.graphs = (bool(graphs) and os.environ.get("EDGE_INFER_ENABLE_QWEN3_GRAPH", "1") != "0"
+                       and model.capture_safe())
         self._captured: Dict[Tuple[int, int], _CapturedDecode] = {}
         self.graph_replays = 0
 

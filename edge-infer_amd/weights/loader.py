@@ -10,6 +10,7 @@ inside the model folder; nothing is ever downloaded.
 from __future__ import annotations
 
 import json
+import os
 from dataclasses import dataclass, field
 from pathlib import Path
 from typing import Dict, List, Mapping, Optional, Tuple
@@ -88,11 +89,15 @@ def read_tensors(model_dir) -> Dict[str, torch.Tensor]:
             shards.setdefault(_shard_path(root, shard), []).append(name)
     else:
         shards = {_shard_path(root, "model.safetensors"): None}
+    # EDGE_INFER_VERBOSE_WEIGHTS=1 lists what is read, as in frontend/checkpoint.py:88-99
+    verbose = os.environ.get("EDGE_INFER_VERBOSE_WEIGHTS") == "1"
     tensors: Dict[str, torch.Tensor] = {}
     for path, names in shards.items():
         with safe_open(str(path), framework="pt", device="cpu") as source:
             for name in (source.keys() if names is None else names):
                 tensors[name] = _stored_precision(source.get_tensor(name))
+                if verbose:
+                    print(f"Loaded {name}: {tuple(tensors[name].shape)}, {tensors[name].dtype}")
     if not tensors:
         raise ValueError("the checkpoint holds no tensors")
     return tensors

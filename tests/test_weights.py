@@ -119,3 +119,16 @@ def test_parameter_inventory_matches_the_architecture():
     H, V, I, Q, KV, d = 96, 381, 200, 256, 32, 32
     layer = 2 * H + Q * H + 2 * KV * H + H * Q + 2 * d + 3 * I * H
     assert total == 2 * V * H + H + 3 * layer
+
+
+def test_verbose_listing_of_what_is_read(tmp_path, monkeypatch, capsys):
+    """EDGE_INFER_VERBOSE_WEIGHTS=1 lists every tensor as the reference's loader does
+    (frontend/checkpoint.py:88-99); without it nothing is printed."""
+    folder = make_folder("A", tmp_path)
+    read_tensors(folder)
+    assert capsys.readouterr().out == ""
+    monkeypatch.setenv("EDGE_INFER_VERBOSE_WEIGHTS", "1")
+    tensors = read_tensors(folder)
+    lines = capsys.readouterr().out.strip().split("\n")
+    assert len(lines) == len(tensors)
+    assert any(line.startswith("Loaded model.embed_tokens.weight: (256, 64)") for line in lines)
