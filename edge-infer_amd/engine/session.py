@@ -95,6 +95,9 @@ class Session:
                        and model.capture_safe())
         self._captured: Dict[Tuple[int, int], _CapturedDecode] = {}
         self.graph_replays = 0
+        # one generation or reset at a time: a callback that calls back into its own session
+        # is refused, as in the reference (bindings/python/include/python_callback.hpp:16-26)
+        self._busy = False
 
     # -- slots -----------------------------------------------------------
     def begin(self) -> int:
@@ -107,6 +110,8 @@ class Session:
 
     def reset(self) -> None:
         """End every live sequence; allocations are kept."""
+        if self._busy:
+            raise RuntimeError("the session is busy; wait for the current operation to finish")
         torch.cuda.synchronize(self.device)
         self.cache.release_all()
 
@@ -154,10 +159,16 @@ class Session:
             self._streams_used += len(prompts)
         params = SamplingParams(temperature=float(temperature), top_p=float(top_p),
                                 top_k=int(top_k), seed=self.seed if seed is None else int(seed))
-        return generate(self, self._sampler, prompts, vocab_size=spec.vocab_size,
-                        max_length=max_length, max_new_tokens=max_new_tokens, params=params,
-                        stop_ids=stop_ids, callback=callback, max_batch=max_batch,
-                        first_stream=first_stream)
+        if self._busy:
+            raise RuntimeError("the session is busy; wait for the current operation to finish")
+        self._busy = True
+        try:
+            return generate(self, self._sampler, prompts, vocab_size=spec.vocab_size,
+                            max_length=max_length, max_new_tokens=max_new_tokens, params=params,
+                            stop_ids=stop_ids, callback=callback, max_batch=max_batch,
+                            first_stream=first_stream)
+        finally:
+            self._busy = False
 
     def generate(self, input_ids, callback=None, max_length=100, temperature=1.0, top_p=0.9,
                  top_k=1, seed=None):

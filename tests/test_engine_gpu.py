@@ -297,6 +297,27 @@ def test_procedural_interface_generates_like_a_session(folders, oracle):
     api._compat["model"] = api._compat["session"] = None
 
 
+def test_a_session_refuses_a_second_operation_while_one_runs(models):
+    """bindings/python/include/python_callback.hpp:16-26: a callback that generates or resets
+    on its own session is refused; the running generation goes on and ends cleanly."""
+    import edge_infer_amd as ei
+    session = ei.Session(models("A", "float32"), max_tokens=256, max_seqs=2)
+    prompt = requests_for("A", [6], seed=3)[0]
+    refused = []
+
+    def callback(index, token):
+        for action in (lambda: session.generate(prompt, max_length=8), session.reset):
+            with pytest.raises(RuntimeError, match="busy"):
+                action()
+            refused.append(token)
+    out = session.generate_batch([prompt], max_new_tokens=3, temperature=0.0, stop_ids=(),
+                                 callback=callback)[0]
+    assert len(out) == 3 and len(refused) == 6
+    assert session.generate_batch([prompt], max_new_tokens=3, temperature=0.0, stop_ids=())[0] == out
+    session.reset()
+    assert session.cache.slots.n_free == 2
+
+
 def test_seeded_sampling_is_the_same_alone_and_in_a_batch(folders, oracle):
     """Configuration B's workload: temperature 0.8 with a seeded sampler.  Every drawn
     token equals the plain sampler's draw from the plain logits of the same prefix."""
