@@ -343,6 +343,37 @@ def test_seeded_sampling_is_the_same_alone_and_in_a_batch(folders, oracle):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_head_size_64_with_groups_of_eight(tmp_path, dtype):
+    """A third shape, for the matrix-core attention at head size 64: 16 query heads on 2 kv
+    heads (decode blocks of 16 waves then take a group in two blocks), an intermediate size
+    that is no multiple of 16 (gate and up stay halves), an odd vocabulary; whole prompts of
+    unequal lengths, then token by token."""
+    import edge_infer_amd as ei
+    cfg = ei.Qwen3Config(vocab_size=777, hidden_size=192, num_hidden_layers=2,
+                         num_attention_heads=16, num_key_value_heads=2, head_dim=64,
+                         intermediate_size=296, max_position_embeddings=512, bos_token_id=0,
+                         eos_token_id=776, rms_norm_eps=1e-5, rope_theta=50000.0,
+                         tie_word_embeddings=True)
+    folder = ei.write_model_folder(tmp_path / "d64", cfg, seed=8)
+    pcfg, pw = plain.read_folder(folder)
+    prompts = [random_ids(777, n, 40 + n) for n in (150, 31, 260)]
+    refs = [plain.forward(pw, pcfg, ids) for ids in prompts]
+    session = ei.Session(ei.load_model(folder, dtype=dtype), max_tokens=1024, max_seqs=3)
+    slots = [session.begin() for _ in prompts]
+    cuts = [len(p) - 12 for p in prompts]
+    logits = session.step([(s, p[:c], [c - 1]) for s, p, c in zip(slots, prompts, cuts)])
+    rows = [[logits[i]] for i in range(3)]
+    for t in range(12):
+        out = session.step([(s, [p[c + t]], [0]) for s, p, c in zip(slots, prompts, cuts)])
+        for i in range(3):
+            rows[i].append(out[i])
+    for i in range(3):
+        assert_close(dtype, torch.stack(rows[i]), refs[i][cuts[i] - 1:], f"d64 {dtype} request {i}")
+    if dtype == "bfloat16":
+        assert session.graph_replays > 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_one_layer_of_the_8b_shape(tmp_path, dtype):
     """Layer sizes of Qwen3-8B (hidden 4096, 32 heads, 8 kv heads, head_dim 128,
     intermediate 12288) with one layer and a small vocabulary: the kernels that the big
