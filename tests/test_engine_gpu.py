@@ -374,6 +374,34 @@ def test_head_size_64_with_groups_of_eight(tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_widths_that_are_no_multiple_of_eight(tmp_path, dtype):
+    """Hidden size 100, intermediate size 52, vocabulary 99: the few-rows product needs a K
+    that is a multiple of 8 and is not taken here (the library multiplies, decode is not
+    captured); the row-wise kernels take their scalar forms.  Results are the same."""
+    import edge_infer_amd as ei
+    cfg = ei.Qwen3Config(vocab_size=99, hidden_size=100, num_hidden_layers=2,
+                         num_attention_heads=3, num_key_value_heads=1, head_dim=16,
+                         intermediate_size=52, max_position_embeddings=128, bos_token_id=0,
+                         eos_token_id=98, rms_norm_eps=1e-6, rope_theta=10000.0,
+                         tie_word_embeddings=False)
+    folder = ei.write_model_folder(tmp_path / "odd", cfg, seed=12)
+    pcfg, pw = plain.read_folder(folder)
+    prompts = [random_ids(99, n, 60 + n) for n in (70, 9)]
+    refs = [plain.forward(pw, pcfg, ids) for ids in prompts]
+    session = ei.Session(ei.load_model(folder, dtype=dtype), max_tokens=256, max_seqs=2)
+    slots = [session.begin() for _ in prompts]
+    cuts = [len(p) - 5 for p in prompts]
+    logits = session.step([(s, p[:c], [c - 1]) for s, p, c in zip(slots, prompts, cuts)])
+    rows = [[logits[i]] for i in range(2)]
+    for t in range(5):
+        out = session.step([(s, [p[c + t]], [0]) for s, p, c in zip(slots, prompts, cuts)])
+        for i in range(2):
+            rows[i].append(out[i])
+    for i in range(2):
+        assert_close(dtype, torch.stack(rows[i]), refs[i][cuts[i] - 1:], f"odd {dtype} request {i}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_one_layer_of_the_8b_shape(tmp_path, dtype):
     """Layer sizes of Qwen3-8B (hidden 4096, 32 heads, 8 kv heads, head_dim 128,
     intermediate 12288) with one layer and a small vocabulary: the kernels that the big
