@@ -123,8 +123,12 @@ def test_swiglu_with_gate_and_up_in_strips(lib, dtype, I, strip):
         lib.swiglu(mixed.contiguous(), out, 7)
 
 
-@pytest.mark.parametrize("shape", [(1, 381, 96), (5, 64, 200), (70, 130, 33), (130, 257, 512)])
+@pytest.mark.parametrize("shape", [(1, 381, 96), (5, 64, 200), (70, 130, 33), (130, 257, 512),
+                                   (8, 100, 1000), (40, 4100, 1028), (6, 77, 260)])
 def test_gemm_f32(lib, shape):
+    """Few rows take the weight-streaming kernel (K in fours), many the tiled one; both sum
+    every output over k in ascending order, so a row gives the same bits alone, among up to
+    8 rows and among many."""
     M, N, K = shape
     a = torch.randn(M, K, device=DEV)
     w = torch.randn(N, K, device=DEV)
@@ -135,6 +139,11 @@ def test_gemm_f32(lib, shape):
     single = torch.empty(1, N, device=DEV)
     lib.gemm_f32(a[M // 2:M // 2 + 1].contiguous(), w, single)
     assert torch.equal(single[0], out[M // 2])
+    for rows in (3, 5, 8):
+        if rows <= M:
+            few = torch.full((rows, N), float("nan"), device=DEV)
+            lib.gemm_f32(a[:rows].contiguous(), w, few)
+            assert torch.equal(few, out[:rows]), rows
 
 
 # ---------------------------------------------------------------------------
