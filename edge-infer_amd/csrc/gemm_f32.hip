@@ -5,8 +5,9 @@
 //
 // Every output element is accumulated over k in ascending order by one thread, so a
 // row's result does not depend on which other rows are in the batch, nor on which of the
-// two kernels below computed it: the tiled one for many rows, the weight-streaming one for
-// up to 8 rows (decode), which reads every weight row in kilobyte pieces.
+// kernels below computed it: two tiled ones (64 x 64 outputs a block; 128 x 128 for many rows
+// with K in fours) and the weight-streaming one for up to 8 rows (decode), which reads every
+// weight row in kilobyte pieces.
 #include "common.cuh"
 
 namespace {
@@ -58,6 +59,83 @@ gemm_f32_kernel(const float* __restrict__ A, const float* __restrict__ W, float*
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
       const int n = n0 + tx * TN + j;
+      if (n < N) C[static_cast<size_t>(m) * ldc + n] = acc[i][j];
+    }
+  }
+}
+
+// Many rows (prefill): tiles of 128 x 128 outputs, 8 x 8 of them a thread (as two by two
+// groups of 4 x 4, so that LDS is read in 16-byte pieces), the next K-tile on its way in
+// registers while this one is multiplied.  The same sums in the same order as above.
+constexpr int GM = 128, GN = 128, GK = 16, GS = GM + 4;
+
+__global__ void __launch_bounds__(256)
+gemm_f32_large_kernel(const float* __restrict__ A, const float* __restrict__ W,
+                      float* __restrict__ C, int M, int N, int K, long long lda, long long ldw,
+                      long long ldc) {
+  typedef float f32x4 __attribute__((ext_vector_type(4)));
+  __shared__ __attribute__((aligned(16))) float As[GK * GS];
+  __shared__ __attribute__((aligned(16))) float Ws[GK * GS];
+  const int t = threadIdx.x, ty = t / 16, tx = t % 16;
+  const int m0 = blockIdx.y * GM, n0 = blockIdx.x * GN;
+  const f32x4 zero = f32x4{0.f, 0.f, 0.f, 0.f};
+  float acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = 0.f;
+  // thread -> two 16-byte pieces of each tile: row f / 4, floats 4 (f % 4) .. + 3, f = t, t + 256
+  f32x4 a_next[2], w_next[2];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int f = t + 256 * i, row = f / 4, k = k0 + 4 * (f % 4);
+      a_next[i] = (m0 + row < M && k < K)
+                      ? *reinterpret_cast<const f32x4*>(A + static_cast<size_t>(m0 + row) * lda + k)
+                      : zero;
+      w_next[i] = (n0 + row < N && k < K)
+                      ? *reinterpret_cast<const f32x4*>(W + static_cast<size_t>(n0 + row) * ldw + k)
+                      : zero;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += GK) {
+    __syncthreads();                      // the previous tile has been read
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int f = t + 256 * i, row = f / 4, kq = 4 * (f % 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        As[(kq + e) * GS + row] = a_next[i][e];
+        Ws[(kq + e) * GS + row] = w_next[i][e];
+      }
+    }
+    __syncthreads();
+    if (k0 + GK < K) fetch(k0 + GK);
+#pragma unroll
+    for (int k = 0; k < GK; ++k) {
+      const f32x4 a0 = *reinterpret_cast<const f32x4*>(&As[k * GS + ty * 4]);
+      const f32x4 a1 = *reinterpret_cast<const f32x4*>(&As[k * GS + 64 + ty * 4]);
+      const f32x4 w0 = *reinterpret_cast<const f32x4*>(&Ws[k * GS + tx * 4]);
+      const f32x4 w1 = *reinterpret_cast<const f32x4*>(&Ws[k * GS + 64 + tx * 4]);
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[i][j] = fmaf(a0[i], w0[j], acc[i][j]);
+          acc[i][4 + j] = fmaf(a0[i], w1[j], acc[i][4 + j]);
+          acc[4 + i][j] = fmaf(a1[i], w0[j], acc[4 + i][j]);
+          acc[4 + i][4 + j] = fmaf(a1[i], w1[j], acc[4 + i][4 + j]);
+        }
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int m = m0 + (i / 4) * 64 + ty * 4 + i % 4;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int n = n0 + (j / 4) * 64 + tx * 4 + j % 4;
       if (n < N) C[static_cast<size_t>(m) * ldc + n] = acc[i][j];
     }
   }
@@ -146,6 +224,13 @@ extern "C" int ei_gemm_f32(const float* A, const float* W, float* C, int M, int 
       gemm_f32_few_rows_kernel<1><<<blocks, EI_WAVE, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc);
     else
       gemm_f32_few_rows_kernel<2><<<blocks, EI_WAVE, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc);
+    EI_LAUNCH_CHECK();
+  }
+  if (M > 64 && fours) {
+    const long long rows = (M + GM - 1) / GM;
+    EI_REQUIRE(rows <= 65535, "gemm_f32: too many rows for one launch");
+    dim3 tiles((N + GN - 1) / GN, static_cast<unsigned>(rows));
+    gemm_f32_large_kernel<<<tiles, 256, 0, stream>>>(A, W, C, M, N, K, lda, ldw, ldc);
     EI_LAUNCH_CHECK();
   }
   const long long gy = (M + BM - 1) / BM;

@@ -124,7 +124,7 @@ def test_swiglu_with_gate_and_up_in_strips(lib, dtype, I, strip):
 
 
 @pytest.mark.parametrize("shape", [(1, 381, 96), (5, 64, 200), (70, 130, 33), (130, 257, 512),
-                                   (8, 100, 1000), (40, 4100, 1028), (6, 77, 260)])
+                                   (8, 100, 1000), (40, 4100, 1028), (6, 77, 260), (200, 300, 264)])
 def test_gemm_f32(lib, shape):
     """Few rows take the weight-streaming kernel (K in fours), many the tiled one; both sum
     every output over k in ascending order, so a row gives the same bits alone, among up to
