@@ -229,7 +229,7 @@ def test_refused_steps_change_nothing(models):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", NAMES)
 def test_greedy_generation_through_the_entry_point(folders, oracle, name, dtype):
-    """BASELINE workload of the tiny configurations: a batch of unequal prompts, then
+    """The workload of the tiny configurations: a batch of unequal prompts, then
     greedy decoding, against the plain implementation that recomputes whole sequences."""
     from edge_infer_amd.api import Model
     cfg, w = oracle[name]
