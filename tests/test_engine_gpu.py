@@ -137,6 +137,38 @@ def test_batches_of_unequal_lengths_one_after_another(models, references, name, 
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_random_schedules_against_the_plain_implementation(models, oracle, dtype):
+    """Seeded random traffic on one session: requests of 1 to 120 tokens in batches of 1 to 4
+    that follow each other on 4 slots and a page budget that is just enough, with tails of
+    random lengths decoded token by token; every returned row against the plain logits."""
+    import random
+    import edge_infer_amd as ei
+    name = "B"
+    cfg, w = oracle[name]
+    rng = random.Random(2024)
+    session = ei.Session(models(name, dtype), max_tokens=4 * 128, max_seqs=4)
+    for tensor in session.cache.kv_k + session.cache.kv_v:
+        tensor.fill_(float("nan"))
+    cache = {}
+    for scenario in range(6):
+        n = rng.randint(1, 4)
+        lengths = [rng.randint(1, 120) for _ in range(n)]
+        requests = [random_ids(cfg["vocab_size"], length, 1000 * scenario + i)
+                    for i, length in enumerate(lengths)]
+        tail = rng.choice([0, 1, 7, 40])
+        got = run_batches(session, requests, [list(range(n))], tail=tail)
+        for r, rows in got.items():
+            key = tuple(requests[r])
+            if key not in cache:
+                cache[key] = plain.forward(w, cfg, requests[r])
+            cut = max(1, len(requests[r]) - tail)
+            assert_close(dtype, rows, cache[key][cut - 1:],
+                         f"{dtype} scenario {scenario} request {r} of lengths {lengths} tail {tail}")
+        assert session.cache.slots.n_free == 4
+    assert all(pool.n_free == pool.n_pages for pool in session.cache.kv_pools)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_batch_composition_changes_nothing(models, dtype):
     """The same request alone and inside two different batches: in float32 the rows are
     bit-identical (every kernel reduces in an order that ignores the neighbours)."""
