@@ -43,8 +43,9 @@ def load_model(model_dir, dtype="bfloat16", device="cuda"):
     return model
 
 
-def random_model(cfg, seed, dtype="bfloat16", device="cuda"):
-    """A model of configuration `cfg` with random weights drawn on the device."""
+def random_model(cfg, seed, dtype="bfloat16", device="cuda", biases=False):
+    """A model of configuration `cfg` with random weights drawn on the device (`biases`:
+    with the optional bias of every projection and of the head)."""
     from .engine.model import DecoderModel, expected_parameters
     from .weights import random_parameters
 
@@ -52,7 +53,7 @@ def random_model(cfg, seed, dtype="bfloat16", device="cuda"):
     spec = cfg.model_spec()
     expected = expected_parameters(spec, cfg.checkpoint_name)
     skip = ("head.weight",) if spec.tie_word_embeddings else ()
-    params = random_parameters(expected, seed, device=device, skip=skip)
+    params = random_parameters(expected, seed, device=device, skip=skip, biases=biases)
     model = DecoderModel(spec, params, dtype, device)
     model.config = cfg
     return model

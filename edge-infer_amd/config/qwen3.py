@@ -186,6 +186,8 @@ class Qwen3Config:
             return "model.norm.weight"
         if parameter == "head.weight":
             return "lm_head.weight"
+        if parameter == "head.bias":
+            return "lm_head.bias"
         parts = parameter.split(".")
         if parts[0] == "layers" and len(parts) >= 4:
             prefix = f"model.layers.{parts[1]}."
@@ -203,9 +205,13 @@ class Qwen3Config:
                 "ffn.up_proj.weight": "mlp.up_proj.weight",
                 "ffn.down_proj.weight": "mlp.down_proj.weight",
             }
+            for path, name in list(table.items()):      # the optional bias of each projection
+                if "_proj." in path:
+                    table[path[:-len("weight")] + "bias"] = name[:-len("weight")] + "bias"
             if rest in table:
                 return prefix + table[rest]
         raise KeyError(f"Qwen3 has no checkpoint tensor for parameter '{parameter}'")
 
     # alternative checkpoint names that mean the same parameter
-    checkpoint_aliases = {"model.lm_head.weight": "lm_head.weight"}
+    checkpoint_aliases = {"model.lm_head.weight": "lm_head.weight",
+                          "model.lm_head.bias": "lm_head.bias"}

@@ -29,6 +29,7 @@ _SIGNATURES = {
         "ei_swiglu": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_int, c_int, c_int, c_int,
                       c_void_p],
         "ei_sum_slices": [c_void_p, c_int, c_longlong, c_void_p, c_longlong, c_void_p],
+        "ei_bias_rows": [c_void_p, c_void_p, c_longlong, c_int, c_int, c_void_p],
     },
     "rope_store": {
         "ei_qk_norm_rope_store": [c_void_p, c_int, c_int, c_longlong, c_void_p, c_void_p, c_float,
@@ -203,6 +204,16 @@ def sum_slices(slices: torch.Tensor, out: torch.Tensor) -> None:
     status = lib.ei_sum_slices(_gpu(slices, "slices", torch.float32), slices.shape[0], n,
                                _gpu(out, "out", torch.float32), n, _stream())
     _check(lib, status, "sum_slices")
+
+
+def bias_rows(bias: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
+    """out[r, :] = bias (accumulate False) or out[r, :] + bias, float32 [rows, width]."""
+    lib = library("rowwise")
+    if out.dim() != 2 or bias.numel() != out.shape[1]:
+        raise KernelError(f"bias_rows: bias of {bias.numel()} for rows {list(out.shape)}")
+    status = lib.ei_bias_rows(_gpu(bias, "bias", torch.float32), _gpu(out, "out", torch.float32),
+                              out.shape[0], out.shape[1], int(accumulate), _stream())
+    _check(lib, status, "bias_rows")
 
 
 def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, eps, rope_table, row_pos, row_seq, page_table,

@@ -222,7 +222,33 @@ __global__ void sum_slices_kernel(const float* __restrict__ in, int nsplit, size
   }
 }
 
+// out[r, j] = bias[j] (+ out[r, j] when `accumulate`): a bias as one more slice of a sliced
+// product, or added to a finished float32 product.
+// operators/src/cuda/execution.cu:61-66,307-317 of the reference (the bias initialises the
+// product's accumulator).
+__global__ void bias_rows_kernel(const float* __restrict__ bias, float* __restrict__ out,
+                                 size_t n, int width, int accumulate) {
+  const size_t start = static_cast<size_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const size_t step = static_cast<size_t>(gridDim.x) * blockDim.x;
+  for (size_t i = start; i < n; i += step) {
+    const float b = bias[i % width];
+    out[i] = accumulate ? out[i] + b : b;
+  }
+}
+
 }  // namespace
+
+extern "C" int ei_bias_rows(const float* bias, float* out, long long rows, int width,
+                            int accumulate, hipStream_t stream) {
+  EI_REQUIRE(bias && out && rows > 0 && width > 0, "bias_rows: bad arguments");
+  const size_t n = static_cast<size_t>(rows) * width;
+  const int threads = 256;
+  size_t blocks = (n + threads - 1) / threads;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  bias_rows_kernel<<<static_cast<unsigned>(blocks), threads, 0, stream>>>(bias, out, n, width,
+                                                                         accumulate);
+  EI_LAUNCH_CHECK();
+}
 
 extern "C" int ei_sum_slices(const float* in, int nsplit, long long stride, float* out,
                              long long n, hipStream_t stream) {

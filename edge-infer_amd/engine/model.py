@@ -43,6 +43,7 @@ def model_parameters(spec: ModelSpec) -> Dict[str, ParamSpec]:
     for name, param in final_cls.parameters(spec.final_norm, spec.hidden_size).items():
         params[f"final_norm.{name}"] = param
     params["head.weight"] = ParamSpec((spec.vocab_size, spec.hidden_size))
+    params["head.bias"] = ParamSpec((spec.vocab_size,), optional=True)
     return params
 
 
@@ -60,7 +61,7 @@ class DecoderModel:
         self.dtype = resolve_dtype(dtype)
         self.device = torch.device(device)
         wanted = model_parameters(spec)
-        missing = [p for p in wanted if p not in params
+        missing = [p for p, param in wanted.items() if p not in params and not param.optional
                    and not (p == "head.weight" and spec.tie_word_embeddings)]
         if missing:
             raise KeyError(f"model parameters missing: {missing}")
@@ -79,9 +80,10 @@ class DecoderModel:
                                     {"weight": params["final_norm.weight"]}, self.dtype,
                                     self.device)
         if "head.weight" in params and params["head.weight"] is not params["embed.weight"]:
-            self.head = Linear(params["head.weight"], self.dtype, self.device)
+            self.head = Linear(params["head.weight"], self.dtype, self.device,
+                               bias=params.get("head.bias"))
         else:  # tied: the head is the embedding table itself (no copy: same type and device)
-            self.head = Linear(self.embed, self.dtype, self.device)
+            self.head = Linear(self.embed, self.dtype, self.device, bias=params.get("head.bias"))
 
     def position_table(self, position_spec):
         """One shared encoding object per distinct position spec."""

@@ -5,7 +5,8 @@ encoding -> keys and values stored in the cache -> attention over the cache ->
 output projection.  The order follows the reference's decoder,
 runtime/include/execution/decoder.hpp:121-158.  Three separate checkpoint matrices
 become one [Q + 2 KV, H] matrix when the part is built: each output element is
-still the same dot product.
+still the same dot product.  Each projection may have a bias
+(runtime/include/models/qwen3_model.hpp:386-395: taken if the checkpoint holds it).
 """
 from __future__ import annotations
 
@@ -28,6 +29,10 @@ class Attention:
             "k_proj.weight": ParamSpec((spec.kv_width, hidden)),
             "v_proj.weight": ParamSpec((spec.kv_width, hidden)),
             "o_proj.weight": ParamSpec((hidden, spec.q_width)),
+            "q_proj.bias": ParamSpec((spec.q_width,), optional=True),
+            "k_proj.bias": ParamSpec((spec.kv_width,), optional=True),
+            "v_proj.bias": ParamSpec((spec.kv_width,), optional=True),
+            "o_proj.bias": ParamSpec((hidden,), optional=True),
         }
         if spec.qk_norm:
             params["q_norm.weight"] = ParamSpec((spec.head_dim,), init="norm")
@@ -55,8 +60,15 @@ class Attention:
         self.dtype = dtype
         fused = torch.cat([params["q_proj.weight"], params["k_proj.weight"],
                            params["v_proj.weight"]], dim=0)
-        self.qkv = Linear(fused, dtype, device)
-        self.o = Linear(params["o_proj.weight"], dtype, device)
+        names = ("q_proj", "k_proj", "v_proj")
+        fused_bias = None
+        if any(f"{name}.bias" in params for name in names):   # absent ones count as zero
+            fused_bias = torch.cat([
+                params[f"{name}.bias"] if f"{name}.bias" in params
+                else params[f"{name}.weight"].new_zeros(params[f"{name}.weight"].shape[0])
+                for name in names])
+        self.qkv = Linear(fused, dtype, device, bias=fused_bias)
+        self.o = Linear(params["o_proj.weight"], dtype, device, bias=params.get("o_proj.bias"))
         self.q_norm = self.k_norm = None
         if spec.qk_norm:
             self.q_norm = params["q_norm.weight"].to(device=device, dtype=torch.float32).contiguous()

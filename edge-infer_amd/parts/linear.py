@@ -12,6 +12,11 @@ weight is loaded: decode is bound by how fast the weights can be read, and the
 contiguous copy reads about a fifth faster than rows that lie a power of two apart.  It
 doubles the memory of the linear weights; EDGE_INFER_STREAM_COPY=0 keeps only the stored
 layout and lets the kernel read that.
+
+An optional bias [out] enters the sum before the one rounding, as in the reference
+(operators/src/cuda/execution.cu:307-317 fills the product's accumulator with it): as one
+more float32 slice beside the few-rows kernel's, as the library product's addend, or added
+to the float32 product.
 """
 from __future__ import annotations
 
@@ -26,12 +31,19 @@ STREAM_COPY = os.environ.get("EDGE_INFER_STREAM_COPY", "1") != "0"
 
 
 class Linear:
-    def __init__(self, weight: torch.Tensor, dtype, device):
+    def __init__(self, weight: torch.Tensor, dtype, device, bias: torch.Tensor = None):
         if weight.dim() != 2:
             raise ValueError("a linear weight must be a matrix [out, in]")
         self.weight = weight.to(device=device, dtype=dtype).contiguous()
         self.out_features, self.in_features = self.weight.shape
         self.dtype = dtype
+        self.bias = self.bias_f32 = None
+        if bias is not None:
+            if tuple(bias.shape) != (self.out_features,):
+                raise ValueError(f"a linear bias must be [{self.out_features}], "
+                                 f"got {list(bias.shape)}")
+            self.bias = bias.to(device=device, dtype=dtype).contiguous()
+            self.bias_f32 = self.bias.to(torch.float32)
         self.packed = None
         if dtype == torch.bfloat16 and STREAM_COPY and self.in_features % 8 == 0:
             self.packed = lib.pack_weight(self.weight)
@@ -50,24 +62,36 @@ class Linear:
         if self.dtype == torch.float32:
             out = ctx.buffer(out_name, (rows, self.out_features), torch.float32)
             lib.gemm_f32(x, self.weight, out)
+            if self.bias is not None:
+                lib.bias_rows(self.bias_f32, out, accumulate=True)
             return out
         if lib.skinny_gemm_ok(rows, self.in_features):
             splits = lib.skinny_gemm_splits(rows, self.out_features, self.in_features)
-            out = ctx.buffer(out_name + ".f32", (splits, rows, self.out_features), torch.float32)
-            self._few_rows(x, out)
+            extra = 0 if self.bias is None else 1
+            out = ctx.buffer(out_name + ".f32", (splits + extra, rows, self.out_features),
+                             torch.float32)
+            self._few_rows(x, out[:splits])
+            if extra:
+                lib.bias_rows(self.bias_f32, out[splits], accumulate=False)
             return out
         out = ctx.buffer(out_name, (rows, self.out_features), torch.bfloat16)
-        torch.matmul(x, self.weight.t(), out=out)
+        self._library(x, out)
         return out
+
+    def _library(self, x: torch.Tensor, out: torch.Tensor) -> None:
+        if self.bias is None:
+            torch.matmul(x, self.weight.t(), out=out)
+        else:
+            torch.addmm(self.bias, x, self.weight.t(), out=out)
 
     def forward_gated(self, ctx, x: torch.Tensor, out_name: str):
         """For a weight whose rows alternate, in strips of `lib.GATE_STRIP`, between gate rows
         and their up rows: silu(gate) * up as [N, out/2] of the storage type straight from
         the few-rows kernel, or None where that kernel does not apply (float32, many rows, a
-        shape whose K it would slice); the caller then takes `forward` and the activation
-        kernel."""
+        shape whose K it would slice, a bias); the caller then takes `forward` and the
+        activation kernel."""
         rows = x.shape[0]
-        if (self.dtype != torch.bfloat16 or not lib.skinny_gemm_ok(rows, self.in_features)
+        if (self.dtype != torch.bfloat16 or self.bias is not None or not lib.skinny_gemm_ok(rows, self.in_features)
                 or self.out_features % (2 * lib.GATE_STRIP)
                 or lib.skinny_gemm_splits(rows, self.out_features, self.in_features) != 1):
             return None
@@ -83,6 +107,8 @@ class Linear:
         out = ctx.buffer(out_name, (rows, self.out_features), torch.float32)
         if self.dtype == torch.float32:
             lib.gemm_f32(x, self.weight, out)
+            if self.bias is not None:
+                lib.bias_rows(self.bias_f32, out, accumulate=True)
             return out
         if self.in_features % 8 == 0 and rows <= max(256, SKINNY_ROWS):
             for start in range(0, rows, SKINNY_ROWS):
@@ -96,8 +122,10 @@ class Linear:
                                         torch.float32)
                     self._few_rows(x[start:stop], slices)
                     lib.sum_slices(slices, out[start:stop])
+            if self.bias is not None:
+                lib.bias_rows(self.bias_f32, out, accumulate=True)
             return out
         low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)
-        torch.matmul(x, self.weight.t(), out=low)
+        self._library(x, low)
         out.copy_(low)
         return out

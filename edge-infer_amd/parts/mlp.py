@@ -6,6 +6,7 @@ of 16 rows, the gate rows of 16 outputs followed by their up rows (when I is a m
 16; else all gate rows, then all up rows).  A wave of the few-rows kernel owns 16 rows, so
 neighbouring waves hold a strip's gate and up sums and the kernel can write
 silu(gate) * up itself; otherwise the activation kernel reads the same layout.
+Optional biases (runtime/include/models/qwen3_model.hpp:396-403) follow their rows.
 """
 from __future__ import annotations
 
@@ -25,6 +26,9 @@ class GatedMLP:
             "gate_proj.weight": ParamSpec((spec.intermediate_size, hidden)),
             "up_proj.weight": ParamSpec((spec.intermediate_size, hidden)),
             "down_proj.weight": ParamSpec((hidden, spec.intermediate_size)),
+            "gate_proj.bias": ParamSpec((spec.intermediate_size,), optional=True),
+            "up_proj.bias": ParamSpec((spec.intermediate_size,), optional=True),
+            "down_proj.bias": ParamSpec((hidden,), optional=True),
         }
 
     def __init__(self, spec, hidden, params, dtype, device):
@@ -40,8 +44,19 @@ class GatedMLP:
             both = both.reshape(2 * inter, hidden)
         else:
             both = torch.cat([gate, up], dim=0)
-        self.gate_up = Linear(both, dtype, device)
-        self.down = Linear(params["down_proj.weight"], dtype, device)
+        both_bias = None
+        if "gate_proj.bias" in params or "up_proj.bias" in params:   # an absent one is zero
+            zero = gate.new_zeros(inter)
+            gate_bias = params.get("gate_proj.bias", zero)
+            up_bias = params.get("up_proj.bias", zero)
+            if self.strip:    # the same interleaving as the rows
+                both_bias = torch.stack([gate_bias.reshape(-1, self.strip),
+                                         up_bias.reshape(-1, self.strip)], dim=1).reshape(-1)
+            else:
+                both_bias = torch.cat([gate_bias, up_bias])
+        self.gate_up = Linear(both, dtype, device, bias=both_bias)
+        self.down = Linear(params["down_proj.weight"], dtype, device,
+                           bias=params.get("down_proj.bias"))
 
     def forward(self, ctx, x):
         n = x.shape[0]

@@ -21,9 +21,12 @@ import torch
 @dataclass(frozen=True)
 class ParamSpec:
     """One parameter a part expects.  `init` chooses the random-weights law:
-    "normal" (N(0, 0.02)) for matrices and tables, "norm" (1 + U(-0.1, 0.1))."""
+    "normal" (N(0, 0.02)) for matrices and tables, "norm" (1 + U(-0.1, 0.1)).
+    `optional`: taken when the checkpoint holds it, no error when it does not (the
+    reference's optional projection biases, runtime/include/models/qwen3_model.hpp:371-403)."""
     shape: Tuple[int, ...]
     init: str = "normal"
+    optional: bool = False
 
 
 @dataclass
@@ -124,7 +127,7 @@ def match_parameters(expected: Mapping[str, Tuple[str, ParamSpec]],
     used = set()
     for parameter, (name, spec) in expected.items():
         if name not in available:
-            if parameter in optional:
+            if parameter in optional or spec.optional:
                 continue
             error.missing.append(name)
             continue

@@ -1,6 +1,7 @@
 """Random-weights mode: a model folder (config.json, model.safetensors) from a
 configuration and a seed.  Matrices and tables are N(0, 0.02), norm weights
-1 + U(-0.1, 0.1), stored in bfloat16.  The reference has no such mode (its tests
+1 + U(-0.1, 0.1), stored in bfloat16; optional parameters (biases) are left out unless
+asked for, and then N(0, 0.02) too.  The reference has no such mode (its tests
 build closed-form weights, runtime/tests/qwen3_session_test.cpp:124-172)."""
 from __future__ import annotations
 
@@ -27,17 +28,20 @@ def random_tensor(spec: ParamSpec, generator: torch.Generator, device="cpu",
 
 
 def random_parameters(expected: Mapping[str, Tuple[str, ParamSpec]], seed: int, device="cpu",
-                      dtype=torch.bfloat16, skip=()) -> Dict[str, torch.Tensor]:
-    """parameter path -> tensor, drawn in the order of `expected`."""
+                      dtype=torch.bfloat16, skip=(), biases=False) -> Dict[str, torch.Tensor]:
+    """parameter path -> tensor, drawn in the order of `expected`; optional parameters
+    only with `biases`."""
     generator = torch.Generator(device=device)
     generator.manual_seed(int(seed))
     return {parameter: random_tensor(spec, generator, device, dtype)
-            for parameter, (_, spec) in expected.items() if parameter not in skip}
+            for parameter, (_, spec) in expected.items()
+            if parameter not in skip and (biases or not spec.optional)}
 
 
-def write_model_folder(path, config, seed: int) -> Path:
+def write_model_folder(path, config, seed: int, biases: bool = False) -> Path:
     """Write config.json and model.safetensors for `config` (an architecture's
-    typed configuration) with weights from `seed`.  A tied head is not stored."""
+    typed configuration) with weights from `seed`.  A tied head is not stored.
+    `biases`: every projection and the head get a bias as well."""
     from safetensors.torch import save_file
     from ..engine.model import expected_parameters
 
@@ -46,7 +50,7 @@ def write_model_folder(path, config, seed: int) -> Path:
     spec = config.model_spec()
     expected = expected_parameters(spec, config.checkpoint_name)
     skip = ("head.weight",) if spec.tie_word_embeddings else ()
-    parameters = random_parameters(expected, seed, skip=skip)
+    parameters = random_parameters(expected, seed, skip=skip, biases=biases)
     tensors = {expected[parameter][0]: tensor.contiguous()
                for parameter, tensor in parameters.items()}
     (path / "config.json").write_text(json.dumps(config.to_dict(), indent=2) + "\n")

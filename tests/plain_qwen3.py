@@ -142,31 +142,36 @@ def attention_block(x, w, cfg, layer, positions):
     """RMSNorm -> q/k/v -> per-head q/k RMSNorm -> RoPE -> attention -> o.
 
     runtime/include/execution/decoder.hpp:121-158; the per-head norm comes
-    before the rotation (:125-136) and uses the model's one eps.
+    before the rotation (:125-136) and uses the model's one eps.  Each projection takes
+    a bias when the checkpoint holds one (runtime/include/models/qwen3_model.hpp:386-395).
     """
     p = f"model.layers.{layer}."
     S = x.shape[0]
     nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], head_dim_of(cfg)
     h = rms_norm(x, w[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
-    q = linear(h, w[p + "self_attn.q_proj.weight"]).reshape(S, nq, d)
-    k = linear(h, w[p + "self_attn.k_proj.weight"]).reshape(S, nkv, d)
-    v = linear(h, w[p + "self_attn.v_proj.weight"]).reshape(S, nkv, d)
+    def project(name, heads):
+        return linear(h, w[p + f"self_attn.{name}.weight"],
+                      w.get(p + f"self_attn.{name}.bias")).reshape(S, heads, d)
+
+    q, k, v = project("q_proj", nq), project("k_proj", nkv), project("v_proj", nkv)
     q = rms_norm(q, w[p + "self_attn.q_norm.weight"], cfg["rms_norm_eps"])
     k = rms_norm(k, w[p + "self_attn.k_norm.weight"], cfg["rms_norm_eps"])
     q = rope(q, positions, cfg["rope_theta"])
     k = rope(k, positions, cfg["rope_theta"])
     a = attention(q, k, v, positions)
-    return linear(a.reshape(S, nq * d), w[p + "self_attn.o_proj.weight"])
+    return linear(a.reshape(S, nq * d), w[p + "self_attn.o_proj.weight"],
+                  w.get(p + "self_attn.o_proj.bias"))
 
 
 def feed_forward_block(x, w, cfg, layer):
     """RMSNorm -> gate, up -> silu(gate) * up -> down.
-    runtime/include/execution/decoder.hpp:161-166."""
+    runtime/include/execution/decoder.hpp:161-166; optional biases
+    runtime/include/models/qwen3_model.hpp:396-403."""
     p = f"model.layers.{layer}."
     h = rms_norm(x, w[p + "post_attention_layernorm.weight"], cfg["rms_norm_eps"])
-    g = linear(h, w[p + "mlp.gate_proj.weight"])
-    u = linear(h, w[p + "mlp.up_proj.weight"])
-    return linear(swiglu(g, u), w[p + "mlp.down_proj.weight"])
+    g = linear(h, w[p + "mlp.gate_proj.weight"], w.get(p + "mlp.gate_proj.bias"))
+    u = linear(h, w[p + "mlp.up_proj.weight"], w.get(p + "mlp.up_proj.bias"))
+    return linear(swiglu(g, u), w[p + "mlp.down_proj.weight"], w.get(p + "mlp.down_proj.bias"))
 
 
 def head_dim_of(cfg):
@@ -199,7 +204,7 @@ def forward(w, cfg, ids, positions=None):
         x = x + attention_block(x, w, cfg, layer, positions)
         x = x + feed_forward_block(x, w, cfg, layer)
     y = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
-    return linear(y, head_weight(w, cfg))
+    return linear(y, head_weight(w, cfg), w.get("lm_head.bias"))   # qwen3_model.hpp:371-372
 
 
 # ----------------------------------------------------------------------------

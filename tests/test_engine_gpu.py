@@ -468,3 +468,61 @@ def test_one_layer_of_the_8b_shape(tmp_path, dtype):
     assert_close(dtype, torch.stack(rows_a), ref_a[310:], f"8B-shape layer {dtype} decode a")
     assert_close(dtype, torch.stack(rows_b), ref_b[60:], f"8B-shape layer {dtype} decode b")
     assert session.graph_replays > 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["all", "some"])
+def test_projection_biases(tmp_path, dtype, which):
+    """The optional biases of the projections and of the head
+    (runtime/include/models/qwen3_model.hpp:371-403), made eight times as large as they are
+    drawn so that a dropped or misplaced one shows.  "all": an intermediate size in whole
+    strips of 16 (gate and up rows interleave, and so must their biases).  "some": no v,
+    up or down bias (absent ones count as zero), an intermediate size that keeps gate and up
+    as halves, a tied head with a bias.  A first step of 347 rows goes to the library's
+    product in bfloat16, a second batch of few rows to the weight-streaming kernel; then
+    token by token."""
+    import edge_infer_amd as ei
+    from safetensors.torch import load_file, save_file
+    cfg = ei.Qwen3Config(vocab_size=333, hidden_size=128, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=32,
+                         intermediate_size=208 if which == "all" else 200,
+                         max_position_embeddings=512, bos_token_id=0, eos_token_id=332,
+                         rms_norm_eps=1e-6, rope_theta=10000.0,
+                         tie_word_embeddings=which == "some")
+    folder = ei.write_model_folder(tmp_path / f"biased_{which}", cfg, seed=21, biases=True)
+    path = str(folder / "model.safetensors")
+    tensors = {}
+    for name, tensor in load_file(path).items():
+        if name.endswith(".bias"):
+            if which == "some" and any(part in name for part in ("v_proj", "up_proj", "down_proj")):
+                continue
+            tensor = (tensor.float() * 8).to(tensor.dtype)
+        tensors[name] = tensor
+    assert sum(name.endswith(".bias") for name in tensors) == (15 if which == "all" else 9)
+    save_file(tensors, path, metadata={"format": "pt"})
+    pcfg, pw = plain.read_folder(folder)
+    prompts = [random_ids(333, n, 80 + n) for n in (300, 40, 7, 90, 12)]
+    refs = [plain.forward(pw, pcfg, ids) for ids in prompts]
+    # the biases matter: without them the logits are far off
+    bare = {name: t for name, t in pw.items() if not name.endswith(".bias")}
+    assert (plain.forward(bare, pcfg, prompts[2]) - refs[2]).abs().max() > 0.1 * refs[2].abs().max()
+    session = ei.Session(ei.load_model(folder, dtype=dtype), max_tokens=1024, max_seqs=3)
+    for batch in ([0, 1, 2], [3, 4]):
+        slots = [session.begin() for _ in batch]
+        cuts = [len(prompts[i]) - 5 for i in batch]
+        logits = session.step([(s, prompts[i][:c], [0, c - 1])
+                               for s, i, c in zip(slots, batch, cuts)])
+        rows = {i: [logits[2 * j + 1]] for j, i in enumerate(batch)}
+        for j, (i, c) in enumerate(zip(batch, cuts)):
+            assert_close(dtype, logits[2 * j][None], refs[i][:1], f"biases {which} first row {i}")
+        for t in range(5):
+            out = session.step([(s, [prompts[i][c + t]], [0])
+                                for s, i, c in zip(slots, batch, cuts)])
+            for j, i in enumerate(batch):
+                rows[i].append(out[j])
+        for i, c in zip(batch, cuts):
+            assert_close(dtype, torch.stack(rows[i]), refs[i][c - 1:], f"biases {which} {dtype} {i}")
+        for s in slots:
+            session.end(s)
+    if dtype == "bfloat16":
+        assert session.graph_replays > 0

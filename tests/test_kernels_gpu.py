@@ -687,6 +687,20 @@ def test_gemm_bf16_skinny_refuses_what_it_cannot_run(lib):
         lib.gemm_bf16_skinny_packed(x[:2], lib.pack_weight(w), 48, torch.empty(1, 2, 48, device=DEV))
 
 
+@pytest.mark.parametrize("rows,width", [(1, 7), (5, 96), (300, 1000)])
+def test_bias_rows(lib, rows, width):
+    g = torch.Generator().manual_seed(rows)
+    bias = torch.randn(width, generator=g).cuda()
+    start = torch.randn(rows, width, generator=g).cuda()
+    out = start.clone()
+    lib.bias_rows(bias, out, accumulate=True)
+    assert torch.equal(out, start + bias)
+    lib.bias_rows(bias, out, accumulate=False)
+    assert torch.equal(out, bias.expand(rows, width))
+    with pytest.raises(lib.KernelError):
+        lib.bias_rows(bias[:-1], out, accumulate=False)
+
+
 def test_sum_slices(lib):
     slices = torch.randn(5, 3, 1001, device=DEV)
     out = torch.empty(3, 1001, device=DEV)

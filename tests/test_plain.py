@@ -284,3 +284,13 @@ def test_generate_rules():
     assert len(out) == 5
     again = plain.generate(w, cfg, prompt, max_length=9, stop_ids={out[2]})
     assert again == out[:out.index(out[2])]
+
+
+def test_linear_bias_is_added_to_every_row():
+    """operators/src/cuda/execution.cu:61-66,307-317: the bias row initialises the product."""
+    g = torch.Generator().manual_seed(3)
+    x, w, b = (torch.randn(shape, generator=g, dtype=torch.float64)
+               for shape in ((5, 7), (3, 7), (3,)))
+    expected = torch.nn.functional.linear(x, w, b)
+    assert torch.allclose(plain.linear(x, w, b), expected, atol=1e-12)
+    assert torch.allclose(plain.linear(x, w, b) - plain.linear(x, w), b.expand(5, 3), atol=1e-12)

@@ -22,7 +22,7 @@ def test_random_folder_round_trip(tmp_path):
     assert Qwen3Config.from_dict(json.loads((folder / "config.json").read_text())) == cfg
     tensors = read_tensors(folder)
     params = match_parameters(expected, tensors)
-    assert set(params) == set(expected)
+    assert set(params) == {name for name, (_, spec) in expected.items() if not spec.optional}
     assert all(t.dtype == torch.bfloat16 for t in tensors.values())
     q = params["layers.2.mixer.q_proj.weight"]
     assert tuple(q.shape) == (8 * 32, 96)                 # [out, in] as stored
@@ -61,13 +61,13 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     del tensors["model.layers.1.mlp.up_proj.weight"]
     del tensors["model.norm.weight"]
     tensors["model.layers.7.self_attn.q_proj.weight"] = torch.zeros(2, 2)
-    tensors["model.layers.0.self_attn.q_proj.bias"] = torch.zeros(256)
+    tensors["model.layers.0.self_attn.q_norm.bias"] = torch.zeros(32)
     tensors["model.layers.0.self_attn.k_proj.weight"] = torch.zeros(96, 32)   # transposed
     with pytest.raises(WeightsError) as info:
         match_parameters(expected, tensors)
     error = info.value
     assert sorted(error.missing) == ["model.layers.1.mlp.up_proj.weight", "model.norm.weight"]
-    assert error.unexpected == ["model.layers.0.self_attn.q_proj.bias",
+    assert error.unexpected == ["model.layers.0.self_attn.q_norm.bias",
                                 "model.layers.7.self_attn.q_proj.weight"]
     assert error.wrong_shape == [("model.layers.0.self_attn.k_proj.weight", (32, 96), (96, 32))]
     text = str(error)
@@ -112,9 +112,12 @@ def test_sharded_checkpoint_and_path_containment(tmp_path):
 
 def test_parameter_inventory_matches_the_architecture():
     cfg = tiny_config("B")
-    params = model_parameters(cfg.model_spec())
+    every = model_parameters(cfg.model_spec())
+    params = {name: p for name, p in every.items() if not p.optional}
     per_layer = 11   # 2 norms, q k v o, q_norm k_norm, gate up down
     assert len(params) == 3 + per_layer * cfg.num_hidden_layers
+    # optional: a bias for each of the seven projections of a layer and for the head
+    assert len(every) - len(params) == 7 * cfg.num_hidden_layers + 1
     total = sum(torch.Size(p.shape).numel() for p in params.values())
     H, V, I, Q, KV, d = 96, 381, 200, 256, 32, 32
     layer = 2 * H + Q * H + 2 * KV * H + H * Q + 2 * d + 3 * I * H
@@ -132,3 +135,43 @@ def test_verbose_listing_of_what_is_read(tmp_path, monkeypatch, capsys):
     lines = capsys.readouterr().out.strip().split("\n")
     assert len(lines) == len(tensors)
     assert any(line.startswith("Loaded model.embed_tokens.weight: (256, 64)") for line in lines)
+
+
+def test_optional_biases_are_taken_when_the_checkpoint_holds_them(tmp_path):
+    """runtime/include/models/qwen3_model.hpp:371-403: each projection and the head may have
+    a bias; none is required, a wrong shape is an error, and `model.lm_head.bias` is an
+    alias (bindings/python/include/decoder_weight_mapper.hpp:114-121)."""
+    cfg, expected = expected_for("B")
+    assert cfg.checkpoint_name("layers.1.mixer.k_proj.bias") == \
+        "model.layers.1.self_attn.k_proj.bias"
+    assert cfg.checkpoint_name("layers.0.ffn.down_proj.bias") == "model.layers.0.mlp.down_proj.bias"
+    assert cfg.checkpoint_name("head.bias") == "lm_head.bias"
+    with pytest.raises(KeyError):
+        cfg.checkpoint_name("layers.0.norm1.bias")
+    plain = read_tensors(make_folder("B", tmp_path))
+    assert not any(name.endswith(".bias") for name in plain)
+    folder = write_model_folder(tmp_path / "biased", cfg, 1, biases=True)
+    tensors = read_tensors(folder)
+    # the weights are the ones the same seed gives without biases?  No: the draws interleave;
+    # what is fixed is that every optional tensor is there with its shape
+    params = match_parameters(expected, tensors)
+    assert set(params) == set(expected)
+    assert tuple(params["layers.2.mixer.q_proj.bias"].shape) == (8 * 32,)
+    assert tuple(params["layers.2.ffn.gate_proj.bias"].shape) == (200,)
+    assert tuple(params["head.bias"].shape) == (381,)
+    # some biases only: fine
+    some = {name: t for name, t in tensors.items()
+            if not name.endswith(".bias") or "q_proj" in name}
+    assert "layers.0.mixer.v_proj.bias" not in match_parameters(expected, some)
+    # the alias of the head's bias
+    some["model.lm_head.bias"] = tensors["lm_head.bias"]
+    params = match_parameters(expected, some, aliases=cfg.checkpoint_aliases)
+    assert params["head.bias"] is tensors["lm_head.bias"]
+    # a wrong shape and a bias the model has no use for are reported
+    tensors["model.layers.0.self_attn.o_proj.bias"] = torch.zeros(95, dtype=torch.bfloat16)
+    tensors["model.layers.0.input_layernorm.bias"] = torch.zeros(96, dtype=torch.bfloat16)
+    with pytest.raises(WeightsError) as caught:
+        match_parameters(expected, tensors)
+    assert caught.value.wrong_shape == [("model.layers.0.self_attn.o_proj.bias", (96,), (95,))]
+    assert caught.value.unexpected == ["model.layers.0.input_layernorm.bias"]
+    assert not caught.value.missing
