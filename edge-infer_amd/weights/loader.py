@@ -35,6 +35,7 @@ class WeightsError(ValueError):
     missing: List[str] = field(default_factory=list)
     unexpected: List[str] = field(default_factory=list)
     wrong_shape: List[Tuple[str, Tuple[int, ...], Tuple[int, ...]]] = field(default_factory=list)
+    duplicate: List[str] = field(default_factory=list)   # stored under two of its names
 
     def __str__(self) -> str:
         lines = ["checkpoint does not match the model:"]
@@ -47,6 +48,9 @@ class WeightsError(ValueError):
             lines.append(f"  wrong shapes ({len(self.wrong_shape)}): " + ", ".join(
                 f"{name} expected {list(want)} got {list(got)}"
                 for name, want, got in self.wrong_shape))
+        if self.duplicate:
+            lines.append(f"  stored twice, under a second name as well ({len(self.duplicate)}): "
+                         + ", ".join(self.duplicate))
         return "\n".join(lines)
 
 
@@ -116,13 +120,17 @@ def match_parameters(expected: Mapping[str, Tuple[str, ParamSpec]],
     path -> parameter path it may be taken from when its own tensor is absent
     (a tied output head).  `aliases`: other checkpoint names for the same
     tensor.  Raises one `WeightsError` that lists every missing tensor, every
-    tensor the model has no use for, and every wrong shape.
+    tensor the model has no use for, every wrong shape, and every tensor that is stored
+    under two of its names.
     """
     optional = dict(optional)
     available = {}
-    for name, tensor in tensors.items():
-        available[dict(aliases).get(name, name)] = tensor
     error = WeightsError()
+    for name, tensor in tensors.items():
+        canonical = dict(aliases).get(name, name)
+        if canonical in available:   # bindings/python/include/decoder_weight_mapper.hpp:173
+            error.duplicate.append(canonical)
+        available[canonical] = tensor
     result: Dict[str, torch.Tensor] = {}
     used = set()
     for parameter, (name, spec) in expected.items():
@@ -142,6 +150,6 @@ def match_parameters(expected: Mapping[str, Tuple[str, ParamSpec]],
             if source in result:
                 result[parameter] = result[source]
     error.unexpected = sorted(set(available) - used)
-    if error.missing or error.unexpected or error.wrong_shape:
+    if error.missing or error.unexpected or error.wrong_shape or error.duplicate:
         raise error
     return result

@@ -52,6 +52,12 @@ def test_tied_head_is_not_stored_and_resolves_to_the_embedding(tmp_path):
     params = match_parameters(expected, tensors, optional={"head.weight": "embed.weight"},
                               aliases=cfg.checkpoint_aliases)
     assert params["head.weight"] is tensors["model.lm_head.weight"]
+    # both names at once: which one is meant cannot be known
+    tensors["lm_head.weight"] = torch.ones(256, 64, dtype=torch.bfloat16)
+    with pytest.raises(WeightsError, match="stored twice") as caught:
+        match_parameters(expected, tensors, optional={"head.weight": "embed.weight"},
+                         aliases=cfg.checkpoint_aliases)
+    assert caught.value.duplicate == ["lm_head.weight"]
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
