@@ -1,13 +1,16 @@
 """Decode and prefill throughput of the Qwen3-8B shape with random weights on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
-                    [--shape 8b|0.6b|32b] [--only decode|prefill] [--prompt P]
+                    [--shape 8b|0.6b|32b] [--only decode|prefill|generate] [--prompt P]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
 sampling, and the tokens fed back).  `prefill` is one prompt of 2,048 tokens;
 `roofline` prices the decode step against HBM bandwidth (every weight it uses once,
 plus the cache of the live requests); `points` hold decode at batch 1 and 64.
+`--only generate` times the generation loop instead: a batch of prompts with lengths
+uniform in [64, 2048] that start together, then `--new-tokens` greedy tokens each (the
+workload named for the 0.6B shape, with `--shape 0.6b --batch 32 --context 8192`).
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
 """
@@ -123,6 +126,38 @@ def measure_prefill(model, cfg, repeats=3):
     return 1000.0 * best
 
 
+def measure_generate(model, cfg, batch, context, new_tokens, repeats=2):
+    """Best wall time of `Session.generate_batch` over a batch of unequal prompts, and the
+    time of its prompt step alone."""
+    import random
+    import torch
+    import edge_infer_amd as ei
+    rng = random.Random(5)
+    lengths = [rng.randint(64, 2048) for _ in range(batch)]
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lengths]
+    session = ei.Session(model, max_tokens=batch * context, max_seqs=batch,
+                         max_seq_tokens=context)
+    total = None
+    for _ in range(repeats + 1):
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        out = session.generate_batch(prompts, max_new_tokens=new_tokens, temperature=0.0,
+                                     stop_ids=())
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        total = elapsed if total is None else min(total, elapsed)
+    slots = [session.begin() for _ in range(batch)]
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    session.step([(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)], copy=False)
+    torch.cuda.synchronize()
+    prompt_s = time.perf_counter() - started
+    for s in slots:
+        session.end(s)
+    return total, prompt_s, sum(lengths), sum(len(o) for o in out)
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -137,8 +172,12 @@ def main():
                         help="prompt length before the timed decode steps (with --only decode)")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--skip-points", action="store_true")
-    parser.add_argument("--only", choices=["decode", "prefill"], default=None,
+    parser.add_argument("--only", choices=["decode", "prefill", "generate"], default=None,
                         help="run one workload only and print its figures (for profiling)")
+    parser.add_argument("--context", type=int, default=CONTEXT,
+                        help="tokens a sequence may hold (with --only generate)")
+    parser.add_argument("--new-tokens", type=int, default=256,
+                        help="tokens generated for each prompt (with --only generate)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -160,6 +199,18 @@ def main():
                           "ms_per_step": round(ms_step, 4),
                           "tokens_per_s": round(args.batch * 1000.0 / ms_step, 1),
                           "context": round(context), "GB/s": round(rate, 1)}))
+        return 0
+    if args.only == "generate":
+        total, prompt_s, prompt_tokens, new = measure_generate(model, cfg, args.batch,
+                                                               args.context, args.new_tokens)
+        steps = args.new_tokens - 1          # the first token comes from the prompt step
+        print(json.dumps({"only": "generate", "shape": args.shape, "batch": args.batch,
+                          "prompt_tokens": prompt_tokens, "new_tokens": new,
+                          "total_ms": round(1e3 * total, 1),
+                          "new_tokens_per_s": round(new / total, 1),
+                          "prompt_step_ms": round(1e3 * prompt_s, 1),
+                          "prompt_tokens_per_s": round(prompt_tokens / prompt_s, 1),
+                          "ms_per_decode_step": round(1e3 * (total - prompt_s) / max(1, steps), 4)}))
         return 0
     if args.only == "prefill":
         prefill_ms = measure_prefill(model, cfg)

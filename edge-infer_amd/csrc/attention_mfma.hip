@@ -27,17 +27,40 @@ constexpr float kLowest = -1.0e30f;
 __device__ __forceinline__ float bf16_lo(uint32_t u) { return __uint_as_float(u << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
 
+// What a block needs to make its own queries, and the new key and value of its kv head, from
+// the fused projection (PREP): the work of the separate norm-rotate-store kernel, saved as a
+// launch per layer.  qkv: float32 partial sums [nsplit][rows, (nq + 2 nkv) * D], added in slice
+// order; per-head RMSNorm weights (or null); the rotation table [positions, D] (cosines, then
+// sines; or null); k_store / v_store: the cache pages to write the new key and value to (null:
+// this run of the layer reads a cache that another run wrote, and has no key of its own).
+// Formulas and order as in rope_store.hip (runtime/include/execution/decoder.hpp:125-140).
+struct DecodePrep {
+  const float* qkv;
+  int nsplit;
+  long long split_stride;
+  const float* q_norm_w;
+  const float* k_norm_w;
+  float eps;
+  const float* rope_table;
+  bf16_t* k_store;
+  bf16_t* v_store;
+};
+
 // GB: query heads of the kv group handled by this block (1..16).  W: waves of the block, each
 // taking every W-th tile of 16 keys of the block's key range: 4 where sequences and slices
 // give many blocks, 16 where they give few (a short range then needs no slices at all).
-template <int D, int GB, int W>
+// PREP: q is not read; the block forms its queries and the position's key and value itself
+// (the block of slice 0 and head block 0 stores them; the wave that meets the position in
+// its tile takes them from LDS, since the store of another block may not have landed).
+template <int D, int GB, int W, bool PREP>
 __global__ void __launch_bounds__(W * EI_WAVE)
 attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                    const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ row_pos,
                    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table,
                    int table_width, bf16_t* __restrict__ out, float* __restrict__ part_o,
                    float* __restrict__ part_ml, int nq, int nkv, int head_blocks, int window,
-                   float scale, int n_splits, const int32_t* __restrict__ longest) {
+                   float scale, int n_splits, const int32_t* __restrict__ longest,
+                   DecodePrep prep) {
   constexpr int DJ = D / 32;            // MFMA steps over the head dimension
   constexpr int LPR = D / 8;            // lanes that cover one value row with 16-byte loads
   constexpr int KPI = EI_WAVE / LPR;    // value rows per load instruction
@@ -59,14 +82,97 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   const int head0 = g * G + hb * GB;               // first query head of this block
   const int heads_here = min(GB, G - hb * GB);
 
+  // PREP: rows 0..GB-1 the block's query heads, row GB the new key, row GB+1 the new value,
+  // normed, rotated and rounded.  A wave takes a head at a time, a lane the pair (i, i + D/2):
+  // every load of a head is on its way before the first is used, and nothing but the final
+  // rows goes through LDS.
+  constexpr int PR = PREP ? GB + 2 : 1, FS = PREP ? D + 8 : 8;
+  __shared__ __attribute__((aligned(16))) bf16_t fin_lds[PR][FS];
+  const bool own_key = PREP && prep.k_store != nullptr;
+  if constexpr (PREP) {
+    constexpr int half = D / 2;
+    static_assert(half <= EI_WAVE, "a lane holds one pair");
+    const size_t width = static_cast<size_t>(nq + 2 * nkv) * D;
+    const float* src = prep.qkv + static_cast<size_t>(row) * width;
+    const int page_now = own_key
+        ? page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE] : -1;
+    const bool active = lane < half;
+    const int i = active ? lane : 0;
+    for (int h = wave; h < heads_here + (own_key ? 2 : 0); h += W) {
+      const int kind = h < heads_here ? 0 : (h == heads_here ? 1 : 2);   // query, key, value
+      const int slot = kind == 0 ? h : GB + kind - 1;
+      const int column = kind == 0 ? (head0 + h) * D
+                                   : (kind == 1 ? (nq + g) * D : (nq + nkv + g) * D);
+      const float* norm_w = kind == 0 ? prep.q_norm_w : (kind == 1 ? prep.k_norm_w : nullptr);
+      const bool rotate = kind != 2 && prep.rope_table != nullptr;
+      float wx = 1.f, wy = 1.f, cs = 1.f, sn = 0.f;
+      if (norm_w != nullptr) {
+        wx = norm_w[i];
+        wy = norm_w[i + half];
+      }
+      if (rotate) {
+        const float* trig = prep.rope_table + static_cast<size_t>(pos) * D;
+        cs = trig[i];
+        sn = trig[i + half];
+      }
+      float x = 0.f, y = 0.f;
+      const float* p = src + column + i;
+      for (int s0 = 0; s0 < prep.nsplit; s0 += 8) {       // slices in slice order, 8 per trip
+        float xa[8], ya[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < prep.nsplit) {
+            xa[u] = p[(s0 + u) * prep.split_stride];
+            ya[u] = p[(s0 + u) * prep.split_stride + half];
+          }
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (s0 + u < prep.nsplit) {
+            x += xa[u];
+            y += ya[u];
+          }
+      }
+      if (!active) x = y = 0.f;
+      float a = x, b = y;
+      if (norm_w != nullptr) {
+        const float sum = ei::wave_sum(x * x + y * y);
+        const float inv = rsqrtf(sum / static_cast<float>(D) + prep.eps);
+        a = (a * inv) * wx;
+        b = (b * inv) * wy;
+      }
+      if (rotate) {
+        const float ra = a * cs - b * sn;
+        const float rb = a * sn + b * cs;
+        a = ra;
+        b = rb;
+      }
+      if (active) {
+        const bf16_t a16 = ei::from_f32<bf16_t>(a), b16 = ei::from_f32<bf16_t>(b);
+        fin_lds[slot][i] = a16;
+        fin_lds[slot][i + half] = b16;
+        if (kind != 0 && hb == 0 && split == 0 && page_now >= 0) {
+          bf16_t* dst = (kind == 1 ? prep.k_store : prep.v_store) +
+                        ((static_cast<size_t>(page_now) * nkv + g) * EI_PAGE + pos % EI_PAGE) * D;
+          dst[i] = a16;
+          dst[i + half] = b16;
+        }
+      }
+    }
+    __syncthreads();
+  }
+
   // query heads as the B operand: lane (n = r16, c) holds q[head n][j*32 + c*8 .. +8]
   bf16x8 q_reg[DJ];
 #pragma unroll
   for (int j = 0; j < DJ; ++j) {
     uint4 z = uint4{0u, 0u, 0u, 0u};
-    if (r16 < heads_here)
-      z = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(row) * nq + head0 + r16) * D +
-                                          j * 32 + c * 8);
+    if (r16 < heads_here) {
+      if constexpr (PREP)
+        z = *reinterpret_cast<const uint4*>(&fin_lds[r16][j * 32 + c * 8]);
+      else
+        z = *reinterpret_cast<const uint4*>(q + (static_cast<size_t>(row) * nq + head0 + r16) * D +
+                                            j * 32 + c * 8);
+    }
     q_reg[j] = *reinterpret_cast<bf16x8*>(&z);
   }
 
@@ -118,6 +224,19 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
 #pragma unroll
     for (int i = 0; i < VI; ++i)
       v_reg[i] = *reinterpret_cast<const uint4*>(vp + static_cast<size_t>(i) * KPI * D);
+    if constexpr (PREP) {
+      if (own_key && tile == last_tile) {          // the position's own key and value
+        if (key0 + r16 == pos) {
+#pragma unroll
+          for (int j = 0; j < DJ; ++j)
+            k_reg[j] = *reinterpret_cast<const bf16x8*>(&fin_lds[GB][j * 32 + c * 8]);
+        }
+#pragma unroll
+        for (int i = 0; i < VI; ++i)
+          if (key0 + i * KPI + ks == pos)
+            v_reg[i] = *reinterpret_cast<const uint4*>(&fin_lds[GB + 1][dc * 8]);
+      }
+    }
 
     f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -573,23 +692,23 @@ __global__ void attn_merge_kernel(const float* __restrict__ part_o,
   }
 }
 
-template <int D, int GB>
+template <int D, int GB, bool PREP>
 void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k,
                    const bf16_t* v, const int32_t* row_pos, const int32_t* row_seq,
                    const int32_t* page_table, int table_width, bf16_t* out, float* part_o,
                    float* part_ml, int nq, int nkv, int head_blocks, int window, float scale,
-                   int n_splits, int waves, const int32_t* longest) {
+                   int n_splits, int waves, const int32_t* longest, const DecodePrep& prep) {
   if constexpr (GB <= 4) {               // the caller gives 16 waves at most 4 heads a block
     if (waves == 16) {
-      attn_decode_kernel<D, GB, 16><<<grid, 16 * EI_WAVE, 0, stream>>>(
+      attn_decode_kernel<D, GB, 16, PREP><<<grid, 16 * EI_WAVE, 0, stream>>>(
           q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-          head_blocks, window, scale, n_splits, longest);
+          head_blocks, window, scale, n_splits, longest, prep);
       return;
     }
   }
-  attn_decode_kernel<D, GB, 4><<<grid, 4 * EI_WAVE, 0, stream>>>(
+  attn_decode_kernel<D, GB, 4, PREP><<<grid, 4 * EI_WAVE, 0, stream>>>(
         q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
-        head_blocks, window, scale, n_splits, longest);
+        head_blocks, window, scale, n_splits, longest, prep);
 }
 
 }  // namespace
@@ -660,20 +779,17 @@ extern "C" int ei_attn_decode_mfma_supported(int D, int G) {
   return (D == 64 || D == 128) && G >= 1 ? 1 : 0;
 }
 
-// q, out: [rows, nq, D] bfloat16, one row per sequence (row_seq < 0: padding row);
-// pages: [n_pages, nkv, 64, D]; n_splits > 1 needs part_o [rows, nq, n_splits, D] and
-// part_ml [rows, nq, n_splits, 2] float32.  longest (or null): one int32 on the device, the most
-// tokens that a sequence of this step holds; slices are then that sequence's share for all.
-extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, const void* v_pages,
-                                        const int32_t* row_pos, const int32_t* row_seq,
-                                        const int32_t* page_table, int table_width, void* out,
-                                        float* part_o, float* part_ml, int rows, int nq, int nkv,
-                                        int D, int window, float scale, int n_splits,
-                                        int waves, const int32_t* longest, hipStream_t stream) {
+static int decode_launch(const void* q, const void* k_pages, const void* v_pages,
+                         const int32_t* row_pos, const int32_t* row_seq,
+                         const int32_t* page_table, int table_width, void* out, float* part_o,
+                         float* part_ml, int rows, int nq, int nkv, int D, int window,
+                         float scale, int n_splits, int waves, const int32_t* longest,
+                         const DecodePrep* prep, hipStream_t stream) {
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
   EI_REQUIRE(waves == 4 || waves == 16, "attention_decode: a block has 4 or 16 waves");
   EI_REQUIRE(D == 64 || D == 128, "attention_decode: this kernel takes head_dim 64 or 128");
-  EI_REQUIRE(q && k_pages && v_pages && row_pos && row_seq && page_table && out && table_width > 0,
+  EI_REQUIRE((q || prep) && k_pages && v_pages && row_pos && row_seq && page_table && out &&
+                 table_width > 0,
              "attention_decode: null pointer");
   EI_REQUIRE(n_splits >= 1 && n_splits <= 64, "attention_decode: splits must be between 1 and 64");
   EI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention_decode: split scratch missing");
@@ -690,10 +806,18 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
   const bf16_t* kk = static_cast<const bf16_t*>(k_pages);
   const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
   bf16_t* oo = static_cast<bf16_t*>(out);
+  const DecodePrep none{};
 #define EI_DECODE(DD, GG)                                                                     \
-  launch_decode<DD, GG>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table, table_width,  \
-                        oo, part_o, part_ml, nq, nkv, head_blocks, window, scale, n_splits,   \
-                        waves, longest)
+  do {                                                                                        \
+    if (prep)                                                                                 \
+      launch_decode<DD, GG, true>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table,     \
+                                  table_width, oo, part_o, part_ml, nq, nkv, head_blocks,     \
+                                  window, scale, n_splits, waves, longest, *prep);            \
+    else                                                                                      \
+      launch_decode<DD, GG, false>(grid, stream, qq, kk, vv, row_pos, row_seq, page_table,    \
+                                   table_width, oo, part_o, part_ml, nq, nkv, head_blocks,    \
+                                   window, scale, n_splits, waves, longest, none);            \
+  } while (0)
 #define EI_DECODE_G(DD)            \
   switch (GB) {                    \
     case 1: EI_DECODE(DD, 1); break;   \
@@ -722,4 +846,47 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
                                                       n_splits, total);
   }
   EI_LAUNCH_CHECK();
+}
+
+// q, out: [rows, nq, D] bfloat16, one row per sequence (row_seq < 0: padding row);
+// pages: [n_pages, nkv, 64, D]; n_splits > 1 needs part_o [rows, nq, n_splits, D] and
+// part_ml [rows, nq, n_splits, 2] float32.  longest (or null): one int32 on the device, the most
+// tokens that a sequence of this step holds; slices are then that sequence's share for all.
+extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, const void* v_pages,
+                                        const int32_t* row_pos, const int32_t* row_seq,
+                                        const int32_t* page_table, int table_width, void* out,
+                                        float* part_o, float* part_ml, int rows, int nq, int nkv,
+                                        int D, int window, float scale, int n_splits,
+                                        int waves, const int32_t* longest, hipStream_t stream) {
+  return decode_launch(q, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
+                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, longest,
+                       nullptr, stream);
+}
+
+// The same from the fused projection instead of q: qkv float32 [nsplit][rows, (nq + 2 nkv) * D]
+// (partial sums, added in slice order); the kernel norms and rotates its queries itself and,
+// with write_cache, also the position's key, and stores that key and the value in the pages
+// (so the separate norm-rotate-store kernel is not needed for these rows).  q_norm_w, k_norm_w
+// (float32 [D]) and rope_table (float32 [positions, D]) may each be null.
+extern "C" int ei_attention_decode_mfma_fused(
+    const float* qkv, int nsplit, long long split_stride, const float* q_norm_w,
+    const float* k_norm_w, float eps, const float* rope_table, int write_cache, void* k_pages,
+    void* v_pages, const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table,
+    int table_width, void* out, float* part_o, float* part_ml, int rows, int nq, int nkv, int D,
+    int window, float scale, int n_splits, int waves, const int32_t* longest,
+    hipStream_t stream) {
+  EI_REQUIRE(qkv && nsplit >= 1 && split_stride >= 0, "attention_decode_fused: bad projection");
+  DecodePrep prep{};
+  prep.qkv = qkv;
+  prep.nsplit = nsplit;
+  prep.split_stride = split_stride;
+  prep.q_norm_w = q_norm_w;
+  prep.k_norm_w = k_norm_w;
+  prep.eps = eps;
+  prep.rope_table = rope_table;
+  prep.k_store = write_cache ? static_cast<bf16_t*>(k_pages) : nullptr;
+  prep.v_store = write_cache ? static_cast<bf16_t*>(v_pages) : nullptr;
+  return decode_launch(nullptr, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
+                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, longest,
+                       &prep, stream);
 }

@@ -53,6 +53,11 @@ _SIGNATURES = {
         "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
+        "ei_attention_decode_mfma_fused": [c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_float,
+                                           c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
+                                           c_int, c_int, c_int, c_int, c_float, c_int, c_int,
+                                           c_void_p, c_void_p],
     },
     "gemm_f32": {
         "ei_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_longlong, c_longlong,
@@ -335,6 +340,18 @@ def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, 
     _check(lib, status, "attention_prefill")
 
 
+class DecodeProjection:
+    """What `attention_decode_mfma` needs to make queries, key and value itself: the fused
+    projection as float32 partial sums [slices, rows, (heads + 2 kv heads) * head_dim], the
+    per-head RMSNorm weights (float32 [head_dim], or None), their eps, the rotation table
+    (float32 [positions, head_dim], or None), and whether the position's key and value are
+    stored in the pages."""
+
+    def __init__(self, qkv, q_norm_w, k_norm_w, eps, rope_table, write_cache):
+        self.qkv, self.q_norm_w, self.k_norm_w = qkv, q_norm_w, k_norm_w
+        self.eps, self.rope_table, self.write_cache = eps, rope_table, write_cache
+
+
 def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,
                           n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
                           part_ml=None, waves=4, longest=None) -> None:
@@ -342,11 +359,26 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
     (4 or 16) of a block share its key range tile by tile; 16 suit few sequences (few
     blocks), whose ranges then need fewer slices or none.  `longest` (int32 [1] on the
     device): the most tokens a sequence of the step holds; every sequence's range is then
-    cut into slices of the longest one's share, so that unequal lengths give equal blocks."""
+    cut into slices of the longest one's share, so that unequal lengths give equal blocks.
+    `q` is the queries [rows, heads * head_dim], or a `DecodeProjection`: the kernel then does
+    the work of `qk_norm_rope_store` for its rows as well."""
     lib = library("attention_mfma")
-    n = q.shape[0]
-    if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
+    n = out.shape[0]
+    fused = isinstance(q, DecodeProjection)
+    if tuple(out.shape) != (n, n_heads * head_dim) or (not fused and tuple(q.shape) != tuple(out.shape)):
         raise KernelError("attention_decode: q and out must be [rows, heads * head_dim]")
+    if fused:
+        width = (n_heads + 2 * n_kv_heads) * head_dim
+        if q.qkv.dim() != 3 or tuple(q.qkv.shape[1:]) != (n, width):
+            raise KernelError(f"attention_decode: the projection must be [slices, {n}, {width}], "
+                              f"got {list(q.qkv.shape)}")
+        for name in ("q_norm_w", "k_norm_w"):
+            weight = getattr(q, name)
+            if weight is not None and weight.numel() != head_dim:
+                raise KernelError(f"attention_decode: {name} must have {head_dim} elements")
+        if q.rope_table is not None and (q.rope_table.dim() != 2
+                                         or q.rope_table.shape[1] != head_dim):
+            raise KernelError("attention_decode: rope table must be [positions, head_dim]")
     expect = (n_kv_heads, PAGE_TOKENS, head_dim)
     if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
         raise KernelError(f"attention_decode: pages must be [*, {expect}]")
@@ -358,6 +390,23 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
             raise KernelError("attention_decode: split scratch missing or too small")
     if scale is None:
         scale = head_dim ** -0.5
+    if fused:
+        def opt(tensor, name):
+            return None if tensor is None else _gpu(tensor, name, torch.float32)
+        status = lib.ei_attention_decode_mfma_fused(
+            _gpu(q.qkv, "qkv", torch.float32), q.qkv.shape[0], n * width,
+            opt(q.q_norm_w, "q_norm"), opt(q.k_norm_w, "k_norm"), float(q.eps),
+            opt(q.rope_table, "rope_table"), int(bool(q.write_cache)),
+            _gpu(k_pages, "k_pages", torch.bfloat16), _gpu(v_pages, "v_pages", torch.bfloat16),
+            _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
+            _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
+            _gpu(out, "out", torch.bfloat16),
+            None if part_o is None else _gpu(part_o, "part_o", torch.float32),
+            None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
+            n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves),
+            None if longest is None else _gpu(longest, "longest", torch.int32), _stream())
+        _check(lib, status, "attention_decode")
+        return
     status = lib.ei_attention_decode_mfma(
         _gpu(q, "q", torch.bfloat16), _gpu(k_pages, "k_pages", torch.bfloat16),
         _gpu(v_pages, "v_pages", torch.bfloat16), _gpu(row_pos, "row_pos", torch.int32),

@@ -10,6 +10,8 @@ still the same dot product.  Each projection may have a bias
 """
 from __future__ import annotations
 
+import os
+
 import torch
 
 from ..csrc import lib
@@ -17,6 +19,10 @@ from ..weights.loader import ParamSpec
 from .base import KVRequest
 from .linear import Linear
 from .registry import lookup
+
+# EDGE_INFER_FUSED_DECODE=0: decode steps launch the norm-rotate-store kernel of their own
+# instead of letting the matrix-core decode kernel do that work
+FUSED_DECODE = os.environ.get("EDGE_INFER_FUSED_DECODE", "1") != "0"
 
 
 class Attention:
@@ -94,11 +100,17 @@ class Attention:
         group_index, k_pages, v_pages = ctx.cache.kv(entry.cache)
         page_table = meta.page_table(group_index)
         qkv = self.qkv.forward(ctx, x, "attn.qkv")
-        q = ctx.buffer("attn.q", (n, spec.q_width))
-        lib.qk_norm_rope_store(
-            qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, self.position.table, meta.row_pos,
-            meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads, spec.n_kv_heads,
-            spec.head_dim, write_cache=entry.writes_cache)
+        if (ctx.decode and self.matrix_cores and FUSED_DECODE and qkv.dim() == 3
+                and qkv.dtype == torch.float32):
+            # the decode kernel norms, rotates and stores for its rows itself: one launch less
+            q = lib.DecodeProjection(qkv, self.q_norm, self.k_norm, spec.qk_norm_eps,
+                                     self.position.table, entry.writes_cache)
+        else:
+            q = ctx.buffer("attn.q", (n, spec.q_width))
+            lib.qk_norm_rope_store(
+                qkv, self.q_norm, self.k_norm, spec.qk_norm_eps, self.position.table,
+                meta.row_pos, meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
+                spec.n_kv_heads, spec.head_dim, write_cache=entry.writes_cache)
         out = ctx.buffer("attn.out", (n, spec.q_width))
         if ctx.decode:
             splits, waves = (ctx.decode_plan(spec.n_kv_heads) if self.matrix_cores

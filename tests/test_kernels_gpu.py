@@ -443,6 +443,80 @@ def test_attention_decode_on_the_matrix_cores_window_and_far_key(lib, window):
     close(out, expected, torch.bfloat16)
 
 
+@pytest.mark.parametrize("nq,nkv,D,splits,waves,slices", [
+    (32, 8, 128, 1, 16, 3), (32, 8, 128, 4, 4, 1), (8, 8, 64, 1, 4, 2), (6, 2, 128, 2, 16, 5),
+    (16, 2, 64, 1, 16, 2), (16, 2, 64, 3, 4, 2), (16, 1, 128, 1, 4, 4), (5, 1, 64, 2, 4, 1)])
+@pytest.mark.parametrize("options", ["norm+rope", "bare", "read-only", "window"])
+def test_attention_decode_from_the_projection(lib, nq, nkv, D, splits, waves, slices, options):
+    """The decode kernel that norms, rotates and stores for its rows itself, against the
+    separate norm-rotate-store kernel followed by the same decode kernel: the same output, the
+    same keys and values in the same places of the cache and nothing else touched.  Lengths
+    before the new token around tile and page boundaries; a padding row; group ratios that
+    give one head block, several, and one that is not full; without norm weights and
+    rotation; a run that stores nothing (it reads another run's cache); a window."""
+    theta, eps = 1e4, 1e-5
+    before = [0, 15, 16, 63, 64, 200, 300, 7]
+    N = len(before)
+    write = options != "read-only"
+    window = 50 if options == "window" else None
+    use = options != "bare"
+    torch.manual_seed(nq + D + splits)
+    caches = []
+    for _ in range(2):
+        cache = PagedCache([n + 1 for n in before], nkv, D, torch.bfloat16, seed=2)
+        g = torch.Generator(device=DEV).manual_seed(5)
+        for b, n in enumerate(before):
+            total = n + (0 if write else 1)     # read-only: the position's key is there already
+            if total:
+                cache.put(b, torch.randn(total, nkv, D, device=DEV, generator=g),
+                          torch.randn(total, nkv, D, device=DEV, generator=g))
+        caches.append(cache)
+    width = (nq + 2 * nkv) * D
+    qkv = torch.randn(slices, N, width, device=DEV)
+    row_pos, row_seq = list(before), list(range(N))
+    row_seq[3] = -1                              # a padding row
+    pos = torch.tensor(row_pos, dtype=torch.int32, device=DEV)
+    seq = torch.tensor(row_seq, dtype=torch.int32, device=DEV)
+    qn = (1 + 0.1 * torch.randn(D, device=DEV)) if use else None
+    kn = (1 + 0.1 * torch.randn(D, device=DEV)) if use else None
+    table = rope_table(D, theta, 512) if use else None
+    longest = torch.tensor([301], dtype=torch.int32, device=DEV)
+    outs = []
+    for fused, cache in zip((False, True), caches):
+        out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=torch.bfloat16)
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = torch.full((N * nq * splits * D,), float("nan"), device=DEV)
+            part_ml = torch.full((N * nq * splits * 2,), float("nan"), device=DEV)
+        if fused:
+            q = lib.DecodeProjection(qkv, qn, kn, eps, table, write)
+        else:
+            q = torch.full((N, nq * D), float("nan"), device=DEV, dtype=torch.bfloat16)
+            lib.qk_norm_rope_store(qkv, qn, kn, eps, table, pos, seq, cache.table_dev, q,
+                                   cache.k, cache.v, nq, nkv, D, write_cache=write)
+        lib.attention_decode_mfma(q, cache.k, cache.v, pos, seq, cache.table_dev, out, nq, nkv, D,
+                                  window=window, n_splits=splits, part_o=part_o, part_ml=part_ml,
+                                  waves=waves, longest=longest)
+        outs.append(out)
+    separate, fused = outs
+    assert torch.isnan(fused[3].float()).all() and torch.isnan(separate[3].float()).all()
+    live = [r for r in range(N) if r != 3]
+    assert not torch.isnan(fused[live].float()).any()
+    close(fused[live], separate[live].double().cpu(), torch.bfloat16)
+    # the caches: values equal bit for bit (a copy); keys equal up to the last bit of a
+    # rounding (the sum of squares is added up in another order); NaN sentinels elsewhere
+    bits = lambda t: t.view(torch.int16)
+    assert torch.equal(bits(caches[0].v), bits(caches[1].v))
+    ka, kb = caches[0].k.float(), caches[1].k.float()
+    assert torch.equal(torch.isnan(ka), torch.isnan(kb))
+    there = ~torch.isnan(ka)
+    assert ((ka[there] - kb[there]).abs() <= 2.0 ** -7 * ka[there].abs() + 1e-6).all()
+    if write:
+        for r in live:
+            page = caches[1].table[row_seq[r], row_pos[r] // PAGE]
+            assert not torch.isnan(kb[page, :, row_pos[r] % PAGE]).any()
+
+
 @pytest.mark.parametrize("nq,nkv,D", [(32, 8, 128), (8, 8, 64), (6, 2, 128), (5, 1, 64),
                                       (12, 3, 128), (16, 16, 64), (8, 1, 128), (2, 1, 64)])
 def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D):
