@@ -12,6 +12,8 @@
 // Mathematics as in attention_generic.hip (operators/src/cuda/execution.cu:137-179 and
 // operators/src/cuda/kernels/flash_attention_variable.cu:121-295 of the reference): keys
 // t <= p (and t > p - window), scale 1/sqrt(d) or the given one, float32 softmax.
+#include <type_traits>
+
 #include "common.cuh"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -207,10 +209,14 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
   const int ks = lane / LPR, dc = lane % LPR;       // value rows: key sub-index, 8-wide chunk
 
-  for (int tile = tile_begin + wave; tile < tile_end; tile += W) {
+  // One tile of 16 keys.  OWN: the tile holds the position itself and the block has made its
+  // key and value (PREP): they come from LDS.  That case has code of its own, so that in
+  // every other tile the score product waits for the keys alone and not for a patch.
+  auto process = [&](const int tile, auto own_tag) {
+    constexpr bool OWN = decltype(own_tag)::value;
     const int key0 = tile * kTile;
     const int phys = page_table[static_cast<size_t>(seq) * table_width + key0 / EI_PAGE];
-    if (phys < 0) continue;                        // released by the window: all masked
+    if (phys < 0) return;                          // released by the window: all masked
     const size_t page_base = (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
     const int in_page = key0 % EI_PAGE;
     // keys: A operand, lane (key r16, c) holds k[key][j*32 + c*8 .. +8]
@@ -224,18 +230,16 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
 #pragma unroll
     for (int i = 0; i < VI; ++i)
       v_reg[i] = *reinterpret_cast<const uint4*>(vp + static_cast<size_t>(i) * KPI * D);
-    if constexpr (PREP) {
-      if (own_key && tile == last_tile) {          // the position's own key and value
-        if (key0 + r16 == pos) {
+    if constexpr (OWN) {                           // the position's own key and value
+      if (key0 + r16 == pos) {
 #pragma unroll
-          for (int j = 0; j < DJ; ++j)
-            k_reg[j] = *reinterpret_cast<const bf16x8*>(&fin_lds[GB][j * 32 + c * 8]);
-        }
-#pragma unroll
-        for (int i = 0; i < VI; ++i)
-          if (key0 + i * KPI + ks == pos)
-            v_reg[i] = *reinterpret_cast<const uint4*>(&fin_lds[GB + 1][dc * 8]);
+        for (int j = 0; j < DJ; ++j)
+          k_reg[j] = *reinterpret_cast<const bf16x8*>(&fin_lds[GB][j * 32 + c * 8]);
       }
+#pragma unroll
+      for (int i = 0; i < VI; ++i)
+        if (key0 + i * KPI + ks == pos)
+          v_reg[i] = *reinterpret_cast<const uint4*>(&fin_lds[GB + 1][dc * 8]);
     }
 
     f32x4 s = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -294,6 +298,12 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
+  };
+  for (int tile = tile_begin + wave; tile < tile_end; tile += W) {
+    if (PREP && own_key && tile == last_tile)
+      process(tile, std::integral_constant<bool, PREP>{});
+    else
+      process(tile, std::false_type{});
   }
 
   // sum the partial outputs of the KPI key sub-groups inside the wave
