@@ -158,7 +158,21 @@ class DecoderModel:
 
     # ------------------------------------------------------------------
     def forward(self, ctx) -> torch.Tensor:
-        """Run the rows of `ctx`; float32 logits [wanted rows, vocab]."""
+        """Run the rows of `ctx`; float32 logits [wanted rows, vocab].  The step's buffers
+        are planned by the workspace per shape of step: rows, sequences, wanted rows, kind,
+        and the context bound that fixes the launch shape of decode attention."""
+        workspace = ctx.workspace
+        workspace.start((ctx.n_rows, ctx.n_seqs, ctx.meta.n_want, ctx.decode,
+                         getattr(ctx, "_fixed_context", None)))
+        try:
+            logits = self._forward(ctx)
+        except BaseException:
+            workspace.abort()
+            raise
+        workspace.finish()
+        return logits
+
+    def _forward(self, ctx) -> torch.Tensor:
         spec = self.spec
         meta = ctx.meta
         residual = ctx.buffer("residual", (ctx.n_rows, spec.hidden_size), torch.float32)
@@ -170,4 +184,5 @@ class DecoderModel:
             return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
         hidden = self.final_norm.add_norm(ctx, residual, pending, "final.h", rows=meta.want_rows,
                                           write_residual=False)
+        ctx.release(pending)
         return self.head.forward_f32(ctx, hidden, "logits")

@@ -112,10 +112,10 @@ class Attention:
                 meta.row_pos, meta.row_seq, page_table, q, k_pages, v_pages, spec.n_heads,
                 spec.n_kv_heads, spec.head_dim, write_cache=entry.writes_cache)
         out = ctx.buffer("attn.out", (n, spec.q_width))
+        part_o = part_ml = None
         if ctx.decode:
             splits, waves = (ctx.decode_plan(spec.n_kv_heads) if self.matrix_cores
                              else (ctx.decode_splits(spec.n_kv_heads), 4))
-            part_o = part_ml = None
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
                                     torch.float32)
@@ -145,4 +145,7 @@ class Attention:
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
                               scale=self.scale)
-        return self.o.forward(ctx, out, "attn.o")
+        ctx.release(qkv, None if isinstance(q, lib.DecodeProjection) else q, part_o, part_ml)
+        delta = self.o.forward(ctx, out, "attn.o")
+        ctx.release(out)
+        return delta

@@ -37,24 +37,147 @@ class StateRequest:
 
 
 class Workspace:
-    """Named device buffers that live across steps and only ever grow."""
+    """Named device buffers of a step.
+
+    Without `start` (a part run on its own): one buffer per name that lives across steps
+    and only ever grows.  Between `start(signature)` and `finish()`: the first step of a
+    signature runs on such buffers and records when each value is asked for and when it
+    is `release`d; from that the planner lays the values out in one arena so that values
+    whose lifetimes do not overlap share storage (the reference plans its decoder
+    buffers the same way, runtime/include/execution/decoder.hpp:46-58 over
+    core/include/execution/workspace_plan.hpp); later steps of that signature take their
+    buffers from the arena.  A step that asks for something else than was recorded (a
+    name, an order, a larger size) is served from named buffers from there on and its
+    signature is planned anew next time.  A name that is asked for again while still live
+    stands for the same storage until then, so the earlier value ends there."""
+
+    MAX_PLANS = 32
 
     def __init__(self, device):
         self.device = device
         self._buffers: Dict[str, torch.Tensor] = {}
+        self._arena: Optional[torch.Tensor] = None
+        self._plans: Dict[object, "_StepLayout"] = {}
+        self._signature = None
+        self._layout: Optional["_StepLayout"] = None     # replaying this layout
+        self._events: Optional[list] = None               # recording these events
+        self._cursor = 0
+        self._names: Dict[int, str] = {}                  # data pointer -> name, this step
 
+    # -- one step ------------------------------------------------------------
+    def start(self, signature) -> None:
+        self._signature = signature
+        self._layout = self._plans.get(signature)
+        self._events = [] if self._layout is None else None
+        self._cursor = 0
+        self._names.clear()
+
+    def finish(self) -> None:
+        if self._events is not None:
+            layout = _StepLayout.plan(self._events)
+            if len(self._plans) >= self.MAX_PLANS:
+                self._plans.pop(next(iter(self._plans)))
+            self._plans[self._signature] = layout
+            if self._arena is None or self._arena.numel() < layout.plan.total_bytes:
+                self._arena = torch.empty(max(layout.plan.total_bytes, 256), dtype=torch.uint8,
+                                          device=self.device)
+                for other in self._plans.values():
+                    other.views.clear()               # they pointed into the old arena
+            self._buffers.clear()    # what the step handed out stays alive with its holders
+        self._signature = self._layout = self._events = None
+
+    def abort(self) -> None:
+        """The step failed: nothing of it is kept."""
+        self._signature = self._layout = self._events = None
+
+    def _diverged(self) -> None:
+        """The step does not follow its recording: named buffers from here on."""
+        self._plans.pop(self._signature, None)
+        self._layout = None
+
+    # -- buffers ---------------------------------------------------------------
     def get(self, name: str, shape, dtype) -> torch.Tensor:
         count = 1
         for extent in shape:
             count *= int(extent)
+        layout = self._layout
+        if layout is not None:
+            index = self._cursor
+            if index < len(layout.events) and layout.events[index][0] == name:
+                _, nbytes, key = layout.events[index]
+                if nbytes is not None and count * dtype.itemsize <= nbytes:
+                    self._cursor = index + 1
+                    view = layout.views.get(index)
+                    if view is None or view.dtype != dtype or tuple(view.shape) != tuple(shape):
+                        offset = layout.plan.at(key).offset
+                        raw = self._arena[offset:offset + count * dtype.itemsize]
+                        view = raw.view(dtype).view(*shape)
+                        layout.views[index] = view
+                    self._names[view.data_ptr()] = name
+                    return view
+            self._diverged()
+        if self._events is not None:
+            self._events.append((name, max(count, 1) * dtype.itemsize))
         held = self._buffers.get(name)
         if held is None or held.dtype != dtype or held.numel() < count:
             held = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._buffers[name] = held
+        if self._signature is not None:
+            self._names[held.data_ptr()] = name
         return held[:count].view(*shape)
 
+    def release(self, which) -> None:
+        """The value last asked for under a name (given as the name, or as the tensor that
+        `get` returned) is not read any more.  Anything else is ignored."""
+        if self._signature is None or which is None:
+            return
+        name = which if isinstance(which, str) else self._names.get(which.data_ptr())
+        if name is None:
+            return
+        layout = self._layout
+        if layout is not None:
+            index = self._cursor
+            if index < len(layout.events) and layout.events[index] == (name, None, None):
+                self._cursor = index + 1
+            else:
+                self._diverged()
+        elif self._events is not None:
+            self._events.append((name, None))
+
     def bytes(self) -> int:
-        return sum(b.numel() * b.element_size() for b in self._buffers.values())
+        arena = 0 if self._arena is None else self._arena.numel()
+        return arena + sum(b.numel() * b.element_size() for b in self._buffers.values())
+
+
+class _StepLayout:
+    """The recorded order of a step's requests and releases, and the plan made of it."""
+
+    def __init__(self, events, plan):
+        self.events = events      # (name, bytes, plan key) for a request, (name, None, None)
+        self.plan = plan
+        self.views: Dict[int, torch.Tensor] = {}
+
+    @classmethod
+    def plan(cls, recorded):
+        from ..cache.workspace import WorkspacePlanner
+        planner = WorkspacePlanner()
+        live: Dict[str, list] = {}        # name -> [plan key, bytes, first use]
+        events = []
+        counts: Dict[str, int] = {}
+        for tick, (name, nbytes) in enumerate(recorded):
+            if name in live:              # released, or asked for again: the value ends
+                key, size, first = live.pop(name)
+                planner.add_request(key, size, first, max(first, tick - 1))
+            if nbytes is None:
+                events.append((name, None, None))
+                continue
+            key = f"{name}#{counts.get(name, 0)}"
+            counts[name] = counts.get(name, 0) + 1
+            live[name] = [key, nbytes, tick]
+            events.append((name, nbytes, key))
+        for key, size, first in live.values():    # never released: live to the step's end
+            planner.add_request(key, size, first, len(recorded))
+        return cls(events, planner.build())
 
 
 class StepContext:
@@ -75,3 +198,11 @@ class StepContext:
 
     def buffer(self, name, shape, dtype=None):
         return self.workspace.get(name, shape, self.dtype if dtype is None else dtype)
+
+    def release(self, *buffers) -> None:
+        """These buffers (tensors that `buffer` returned, or their names) are not read any
+        more in this step: their storage may serve a later request.  Optional: what is
+        never released lives to the end of the step; None and tensors that are not the
+        workspace's are ignored."""
+        for which in buffers:
+            self.workspace.release(which)

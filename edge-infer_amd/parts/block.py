@@ -46,6 +46,11 @@ class PreNormBlock:
 
     def forward(self, ctx, residual, pending, entry):
         h = self.norm1.add_norm(ctx, residual, pending, "block.h")
+        ctx.release(pending)             # added into the residual: its storage is free
         a = self.mixer.forward(ctx, h, entry)
+        ctx.release(h)
         h2 = self.norm2.add_norm(ctx, residual, a, "block.h")
-        return self.ffn.forward(ctx, h2)
+        ctx.release(a)
+        out = self.ffn.forward(ctx, h2)
+        ctx.release(h2)
+        return out

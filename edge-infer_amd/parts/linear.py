@@ -122,10 +122,12 @@ class Linear:
                                         torch.float32)
                     self._few_rows(x[start:stop], slices)
                     lib.sum_slices(slices, out[start:stop])
+                    ctx.release(slices)
             if self.bias is not None:
                 lib.bias_rows(self.bias_f32, out, accumulate=True)
             return out
         low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)
         self._library(x, low)
         out.copy_(low)
+        ctx.release(low)
         return out

@@ -65,4 +65,7 @@ class GatedMLP:
             gate_up = self.gate_up.forward(ctx, x, "mlp.gate_up")
             act = ctx.buffer("mlp.act", (n, self.spec.intermediate_size))
             lib.swiglu(gate_up, act, self.strip)
-        return self.down.forward(ctx, act, "mlp.down")
+            ctx.release(gate_up)
+        out = self.down.forward(ctx, act, "mlp.down")
+        ctx.release(act)
+        return out

@@ -526,3 +526,41 @@ def test_projection_biases(tmp_path, dtype, which):
             session.end(s)
     if dtype == "bfloat16":
         assert session.graph_replays > 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_planned_workspace_gives_the_same_logits_in_less_storage(models, references, dtype):
+    """The first step of a shape runs on one buffer per name and records lifetimes; the
+    next step of that shape runs in the planned arena, where dead intermediates share
+    storage: the same logits bit for bit, fewer bytes, and the plan holds no two live values
+    in one place (its constructor checks that)."""
+    import edge_infer_amd as ei
+    session = ei.Session(models("B", dtype), max_tokens=1024, max_seqs=4, graphs=False)
+    prompts = requests_for("B", LENGTHS["B"])[:3]
+    results = []
+    for _ in range(3):
+        slots = [session.begin() for _ in prompts]
+        logits = session.step([(s, p, [0, len(p) - 1]) for s, p in zip(slots, prompts)])
+        tokens = [[1], [2], [3]]
+        decoded = session.step([(s, t, [0]) for s, t in zip(slots, tokens)])
+        results.append((logits, decoded))
+        for s in slots:
+            session.end(s)
+    for logits, decoded in results[1:]:
+        assert torch.equal(logits, results[0][0]) and torch.equal(decoded, results[0][1])
+    for i, p in enumerate(prompts):
+        assert_close(dtype, results[2][0][2 * i + 1][None], references["B"][i][-1:], "planned")
+    plans = list(session.workspace._plans.values())
+    assert len(plans) == 2                                # the prompt step and the decode step
+    for layout in plans:
+        plan = layout.plan
+        assert plan.reused_bytes() > 0 and plan.slot_count() < len(plan.allocations)
+        assert plan.total_bytes < plan.unaliased_bytes()
+    assert session.workspace.bytes() == max(256, max(l.plan.total_bytes for l in plans))
+    # a step that wants no logits plans none (runtime/tests/decoder_output_plan_test.cpp:11-41)
+    slot = session.begin()
+    for _ in range(2):
+        assert session.step([(slot, prompts[0][:7], [])]).shape == (0, 381)
+    silent = [l.plan for sig, l in session.workspace._plans.items() if sig[2] == 0]
+    assert len(silent) == 1 and not any(a.name.startswith("logits") for a in silent[0].allocations)
+    assert any(a.name.startswith("logits") for a in plans[0].plan.allocations)
