@@ -98,10 +98,12 @@ class Session:
         # one generation or reset at a time: a callback that calls back into its own session
         # is refused, as in the reference (bindings/python/include/python_callback.hpp:16-26)
         self._busy = False
+        self._unusable = False     # set for good when a failed step cannot even be waited for
 
     # -- slots -----------------------------------------------------------
     def begin(self) -> int:
         """Take a slot for a new sequence (length 0)."""
+        self._require_usable()
         return self.cache.acquire()
 
     def end(self, slot: int) -> None:
@@ -112,6 +114,7 @@ class Session:
         """End every live sequence; allocations are kept."""
         if self._busy:
             raise RuntimeError("the session is busy; wait for the current operation to finish")
+        self._require_usable()
         torch.cuda.synchronize(self.device)
         self.cache.release_all()
 
@@ -134,6 +137,24 @@ class Session:
     @property
     def max_batch(self) -> int:
         return self.cache.n_slots
+
+    def workspace_report(self) -> dict:
+        """Bytes of the step workspaces: what is held, and for every planned shape of step
+        (rows, sequences, wanted rows, decode, context bound) the arena it needs, what its
+        values would need without sharing, and what sharing saves (the reference reports
+        the same of its decode plan, runtime/include/qwen3.hpp:60-63)."""
+        def plans(workspace):
+            return {signature: {"arena_bytes": layout.plan.total_bytes,
+                                "unaliased_bytes": layout.plan.unaliased_bytes(),
+                                "reused_bytes": layout.plan.reused_bytes(),
+                                "values": len(layout.plan.allocations),
+                                "slots": layout.plan.slot_count()}
+                    for signature, layout in workspace._plans.items()}
+        report = {"held_bytes": self.workspace.bytes(), "plans": plans(self.workspace)}
+        for key, captured in self._captured.items():
+            report["held_bytes"] += captured.workspace.bytes()
+            report["plans"].update(plans(captured.workspace))
+        return report
 
     def free_tokens(self) -> int:
         if not self.cache.kv_pools:
@@ -216,21 +237,41 @@ class Session:
         logits [number of wanted places, vocab] in the order of entries and places.
         With copy=False the result is a view of the session's workspace that the next
         step overwrites."""
+        self._require_usable()
         seqs = self._validate(entries)
         growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
         self.cache.check_growth(growth)          # raises before anything changes
         self.cache.grow(growth)
-        # batches beyond the few-rows product's reach multiply through the library, whose
-        # kernels are kept out of graphs
-        if (self.graphs and len(seqs) <= SKINNY_ROWS
-                and all(seq.count == 1 for seq in seqs)):
-            logits = self._run_captured(seqs)
-        else:
-            plan = StepPlan(seqs, item_sizes=self._item_sizes)
-            logits = self._run(plan, self.meta, self.workspace)
+        try:
+            # batches beyond the few-rows product's reach multiply through the library, whose
+            # kernels are kept out of graphs
+            if (self.graphs and len(seqs) <= SKINNY_ROWS
+                    and all(seq.count == 1 for seq in seqs)):
+                logits = self._run_captured(seqs)
+            else:
+                plan = StepPlan(seqs, item_sizes=self._item_sizes)
+                logits = self._run(plan, self.meta, self.workspace)
+        except BaseException:
+            self._drain_failed_step()
+            raise                                 # the original error
         self.cache.commit(growth)
         self.steps_run += 1
         return logits.clone() if copy else logits
+
+    def _require_usable(self) -> None:
+        if self._unusable:
+            raise RuntimeError("the session is unusable after a failed GPU stream completion")
+
+    def _drain_failed_step(self) -> None:
+        """After an error in a step that may have launched work: wait for what was launched.
+        The sequences keep the lengths they had (what the step wrote lies beyond them and
+        is written again by the next step), so the session stays usable; only if the wait
+        itself fails is nothing known any more, and the session refuses every later call,
+        as the reference's does (runtime/src/qwen3.cpp:126-161,374-379)."""
+        try:
+            torch.cuda.synchronize(self.device)
+        except Exception:       # the original error is the one that is raised
+            self._unusable = True
 
     def _context(self, plan, meta, workspace, fixed_context=None):
         slots = [seq.slot for seq in plan.seqs]
@@ -268,11 +309,15 @@ class Session:
             captured = self._captured[(bucket, bound)] = _CapturedDecode(self.device)
         ctx = self._context(plan, captured.meta, captured.workspace, fixed_context=bound)
         if captured.graph is None:
-            logits = self.model.forward(ctx)
-            torch.cuda.synchronize(self.device)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                captured.logits = self.model.forward(ctx)
+            try:
+                logits = self.model.forward(ctx)
+                torch.cuda.synchronize(self.device)
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph):
+                    captured.logits = self.model.forward(ctx)
+            except BaseException:
+                self._captured.pop((bucket, bound), None)   # nothing half-made is kept
+                raise
             captured.graph = graph
         else:
             captured.graph.replay()

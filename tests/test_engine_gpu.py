@@ -557,6 +557,10 @@ def test_planned_workspace_gives_the_same_logits_in_less_storage(models, referen
         assert plan.reused_bytes() > 0 and plan.slot_count() < len(plan.allocations)
         assert plan.total_bytes < plan.unaliased_bytes()
     assert session.workspace.bytes() == max(256, max(l.plan.total_bytes for l in plans))
+    report = session.workspace_report()
+    assert report["held_bytes"] == session.workspace.bytes() and len(report["plans"]) == 2
+    assert all(p["reused_bytes"] == p["unaliased_bytes"] - p["arena_bytes"] > 0
+               for p in report["plans"].values())
     # a step that wants no logits plans none (runtime/tests/decoder_output_plan_test.cpp:11-41)
     slot = session.begin()
     for _ in range(2):
@@ -564,3 +568,49 @@ def test_planned_workspace_gives_the_same_logits_in_less_storage(models, referen
     silent = [l.plan for sig, l in session.workspace._plans.items() if sig[2] == 0]
     assert len(silent) == 1 and not any(a.name.startswith("logits") for a in silent[0].allocations)
     assert any(a.name.startswith("logits") for a in plans[0].plan.allocations)
+
+
+def test_a_failed_step_leaves_the_session_as_it_was_and_a_failed_wait_ends_it(models, references,
+                                                                              monkeypatch):
+    """The failure contract (runtime/src/qwen3.cpp:126-161,374-379 of the reference), with the
+    failures forced from the host: an error inside a step is raised as it is, the sequences
+    keep their lengths and go on correctly afterwards; if even waiting for the launched work
+    fails, the session refuses every later call."""
+    import edge_infer_amd as ei
+    model = models("A", "float32")
+    session = ei.Session(model, max_tokens=512, max_seqs=2)
+    ids = requests_for("A", LENGTHS["A"])[0]
+    ref = references["A"][0]
+    slot = session.begin()
+    session.step([(slot, ids[:40], [])])
+    real_forward = model.forward
+    calls = []
+
+    def failing(ctx):
+        calls.append(ctx.n_rows)
+        real_forward(ctx)                          # the work is launched, then the step fails
+        raise FloatingPointError("forced")
+    monkeypatch.setattr(model, "forward", failing)
+    for tokens in (ids[40:50], ids[40:41]):        # a prompt chunk and a decode step
+        with pytest.raises(FloatingPointError, match="forced"):
+            session.step([(slot, tokens, [0])])
+        assert session.length(slot) == 40
+    monkeypatch.setattr(model, "forward", real_forward)
+    logits = session.step([(slot, ids[40:50], list(range(10)))])
+    assert_close("float32", logits, ref[40:50], "after failed steps")
+    out = session.step([(slot, ids[50:51], [0])])
+    assert_close("float32", out, ref[50:51], "decode after failed steps")
+    # the wait fails as well: unusable for good
+    monkeypatch.setattr(model, "forward", failing)
+
+    def no_sync(device=None):
+        raise RuntimeError("forced sync failure")
+    monkeypatch.setattr(torch.cuda, "synchronize", no_sync)
+    with pytest.raises(FloatingPointError, match="forced"):
+        session.step([(slot, ids[51:53], [0])])     # (two tokens: a single one would replay a graph)
+    monkeypatch.undo()
+    for call in (lambda: session.step([(slot, ids[51:52], [0])]), session.begin, session.reset,
+                 lambda: session.generate([1, 2, 3])):
+        with pytest.raises(RuntimeError, match="unusable"):
+            call()
+    torch.cuda.synchronize()
