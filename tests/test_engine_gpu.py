@@ -207,6 +207,26 @@ def test_a_batch_wider_than_64_sequences(models, oracle, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_a_decode_batch_beyond_the_few_rows_product(models, oracle, dtype):
+    """260 sequences decode together: more rows than the weight-streaming product takes, so
+    the bfloat16 step multiplies through the library, runs eagerly and prepares queries and
+    keys with the kernel of their own; as sequences end it comes back under 256 rows and
+    to the graphs."""
+    import edge_infer_amd as ei
+    name = "B"
+    cfg, w = oracle[name]
+    lengths = [4 + (5 * i) % 7 for i in range(260)]
+    requests = requests_for(name, lengths, seed=901)
+    session = ei.Session(models(name, dtype), max_tokens=260 * 64, max_seqs=260)
+    got = run_batches(session, requests, [list(range(260))], tail=6)
+    for r in (0, 1, 100, 255, 256, 259):
+        ref = plain.forward(w, cfg, requests[r])
+        cut = max(1, len(requests[r]) - 6)
+        assert_close(dtype, got[r], ref[cut - 1:], f"{dtype} request {r} of a batch of 260")
+    assert session.cache.slots.n_free == 260
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_long_decoding_and_first_tokens(models, oracle, dtype):
     """A prompt of one token, then 230 tokens one by one across three page boundaries."""
     import edge_infer_amd as ei
@@ -374,13 +394,18 @@ def test_seeded_sampling_is_the_same_alone_and_in_a_batch(folders, oracle):
     assert again != together
 
 
+@pytest.mark.parametrize("fused", [True, False])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_head_size_64_with_groups_of_eight(tmp_path, dtype):
+def test_head_size_64_with_groups_of_eight(tmp_path, dtype, fused, monkeypatch):
     """A third shape, for the matrix-core attention at head size 64: 16 query heads on 2 kv
     heads (decode blocks of 16 waves then take a group in two blocks), an intermediate size
     that is no multiple of 16 (gate and up stay halves), an odd vocabulary; whole prompts of
-    unequal lengths, then token by token."""
+    unequal lengths, then token by token.  Decode with the attention kernel making its own
+    queries and keys, and with the separate kernel for that (which batches beyond 256 rows
+    take)."""
     import edge_infer_amd as ei
+    from edge_infer_amd.parts import attention
+    monkeypatch.setattr(attention, "FUSED_DECODE", fused)
     cfg = ei.Qwen3Config(vocab_size=777, hidden_size=192, num_hidden_layers=2,
                          num_attention_heads=16, num_key_value_heads=2, head_dim=64,
                          intermediate_size=296, max_position_embeddings=512, bos_token_id=0,
