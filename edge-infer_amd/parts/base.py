@@ -74,7 +74,7 @@ class Workspace:
 
     def finish(self) -> None:
         if self._events is not None:
-            layout = _StepLayout.plan(self._events)
+            layout = _StepLayout.from_recording(self._events)
             if len(self._plans) >= self.MAX_PLANS:
                 self._plans.pop(next(iter(self._plans)))
             self._plans[self._signature] = layout
@@ -158,7 +158,10 @@ class _StepLayout:
         self.views: Dict[int, torch.Tensor] = {}
 
     @classmethod
-    def plan(cls, recorded):
+    def from_recording(cls, recorded):
+        """recorded: (name, bytes) for each request and (name, None) for each release, in
+        order; a value lives from its request to the event before its release (or before
+        the next request of its name), or to the end."""
         from ..cache.workspace import WorkspacePlanner
         planner = WorkspacePlanner()
         live: Dict[str, list] = {}        # name -> [plan key, bytes, first use]
