@@ -27,7 +27,7 @@ from typing import Mapping, Optional
 import torch
 
 from . import require_gpu
-from .config import read_config, resolve_architecture
+from .config import resolve_architecture
 from .engine.generate import generate  # noqa: F401  (re-exported)
 from .engine.model import DecoderModel, expected_parameters
 from .engine.session import Session

@@ -14,7 +14,7 @@ row_seq = -1, want_rows = -1 and items with seq = -1: kernels skip them.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np

@@ -14,7 +14,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
-from ..cache.allocator import PAGE_TOKENS, CacheFull
+from ..cache.allocator import PAGE_TOKENS
 from ..cache.storage import CacheLayout, SessionCache
 from ..parts.base import StepContext, Workspace
 from ..parts.linear import SKINNY_ROWS

@@ -18,7 +18,6 @@ from ..csrc import lib
 from ..weights.loader import ParamSpec
 from .base import KVRequest
 from .linear import Linear
-from .registry import lookup
 
 # EDGE_INFER_FUSED_DECODE=0: decode steps launch the norm-rotate-store kernel of their own
 # instead of letting the matrix-core decode kernel do that work

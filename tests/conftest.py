@@ -1,8 +1,5 @@
-import os
 import sys
 from pathlib import Path
-
-import pytest
 
 ROOT = Path(__file__).resolve().parents[1]
 for entry in (str(ROOT), str(ROOT / "tests")):

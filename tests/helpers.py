@@ -1,7 +1,5 @@
 """Shared test fixtures: two tiny Qwen3 configurations that differ in every size and
 option, and tolerances that are fixed here once."""
-import json
-import tempfile
 from pathlib import Path
 
 import torch

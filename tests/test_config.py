@@ -8,7 +8,7 @@ from edge_infer_amd.config import (ConfigError, known_architectures, read_config
                                    register_architecture, resolve_architecture,
                                    unregister_architecture)
 from edge_infer_amd.config.specs import ModelSpec, ScheduleEntry
-from helpers import CONFIGS, tiny_config
+from helpers import tiny_config
 
 
 def raw(name, **extra):

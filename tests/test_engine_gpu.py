@@ -1,7 +1,6 @@
 """The engine against the plain implementation, in float32 and in bfloat16: requests
 alone and whole, their last 32 tokens one by one, batches of unequal lengths with slot
 reuse, long decoding, first tokens, generation through the entry point."""
-import numpy as np
 import pytest
 import torch
 

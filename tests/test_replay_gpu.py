@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
-from helpers import assert_close, make_folder, random_ids, tiny_config
+from helpers import assert_close, make_folder, random_ids
 
 pytestmark = pytest.mark.gpu
 ROOT = Path(__file__).resolve().parents[1]
