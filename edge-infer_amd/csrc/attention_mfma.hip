@@ -21,8 +21,6 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int kWaves = 4;
-constexpr int kThreads = kWaves * EI_WAVE;
 constexpr int kTile = 16;          // keys per MFMA tile
 constexpr float kLowest = -1.0e30f;
 
@@ -388,7 +386,6 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   constexpr int KS = D + 8;              // LDS stride of a key row (elements)
   constexpr int VS = EI_PAGE + 4;        // LDS stride of a transposed value row (34 dwords)
   constexpr int CI = D / 64;             // 16-byte chunks per thread per page (D/8 * 64 / 512)
-  constexpr int PW = kPrefillWaves / HB; // waves along the positions
   constexpr int RT = kRowTiles;
   // two pages of keys and of (transposed) values alternate, so that a page costs one barrier
   __shared__ __attribute__((aligned(16))) bf16_t k_lds2[2][EI_PAGE * KS];

@@ -29,12 +29,6 @@ namespace {
 
 constexpr int kPackedTile = 16 * 32;      // elements of one packed tile: 16 rows x 32 k, 1 KB
 
-// Address of the 16-byte piece that lane `lane` takes of the packed tile (kt, strip).
-__device__ __forceinline__ const bf16_t* packed_piece(const bf16_t* Wp, int n_strips, int kt,
-                                                      int strip, int lane) {
-  return Wp + (static_cast<size_t>(kt) * n_strips + strip) * kPackedTile + lane * 8;
-}
-
 // MB * 16 rows of X per workgroup, any K range.  A workgroup is WAVES waves, each owning 16
 // rows of W; X travels through LDS one K-tile (256) at a time, two tiles of it alternate so
 // that a tile costs one barrier.  W has two register sets that are refilled piece by piece:
@@ -54,7 +48,6 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
                    float* __restrict__ out, bf16_t* __restrict__ gated_out, int M, int N, int K,
                    int k_per_split, int row_groups) {
   constexpr int KT = 256, JN = KT / 32;   // MFMA steps per K-tile
-  constexpr int THREADS = WAVES * EI_WAVE;
   constexpr int ROWS_X = MB * 16;
   constexpr int XS = KT;                  // LDS row stride in elements; the 16-byte chunks of a
                                           // row are stored at (chunk ^ row % 16), see store_x

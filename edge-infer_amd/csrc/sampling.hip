@@ -267,7 +267,7 @@ __device__ bool sample_row(const Source<LIST>& source, int k, float top_p, uint6
   if (n_equal_seen <= kMaxTopK) {
     // few ties: the `need_equal` lowest indices by counting smaller ones
     const unsigned count = n_equal_seen;
-    if (t < count) {
+    if (static_cast<unsigned>(t) < count) {
       const int mine = equal_index[t];
       unsigned rank = 0u;
       for (unsigned j = 0; j < count; ++j) rank += equal_index[j] < mine;
