@@ -39,15 +39,27 @@ class _Context(StepContext):
         return max(1, min(wanted, pages, 32))
 
     def decode_plan(self, n_kv_heads: int):
-        """(slices, waves per block) for the matrix-core decode kernel.  Few sequences with
-        contexts up to 2,048: one block of 16 waves per (sequence, kv head) takes the whole
-        key range, a tile of 16 keys per wave at a time, and nothing has to be merged
-        afterwards.  Otherwise blocks of 4 waves over slices of the range, as above (measured
-        faster for long contexts than fewer slices with more waves)."""
+        """(slices, waves per block) for the matrix-core decode kernel.  Up to 256 (sequence,
+        kv head) pairs: blocks of 16 waves, a tile of 16 keys per wave at a time, and as many
+        slices of the key range as shorten a wave's walk by more than the merge kernel costs,
+        while all blocks still fit the chip at once (256 compute units x 16 waves).  The
+        weights are measured ones: 1.9 us for a tile a wave walks, 4.5 us for the merge and
+        0.1 us for each slice it reads.  More pairs than that: blocks of 4 waves, see
+        `decode_splits`."""
         context = self._fixed_context or self.max_context
-        if self.n_seqs * n_kv_heads < 256 and context <= 2048:
-            return 1, 16
-        return self.decode_splits(n_kv_heads), 4
+        pairs = self.n_seqs * n_kv_heads
+        if pairs > 256:
+            return self.decode_splits(n_kv_heads), 4
+        tiles = (context + 15) // 16
+        pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
+        best, best_cost = 1, 1.9 * ((tiles + 15) // 16)
+        slices = 2
+        while slices <= min(pages, 32) and pairs * 16 * slices <= 4096:
+            cost = 1.9 * ((tiles + 16 * slices - 1) // (16 * slices)) + 4.5 + 0.1 * slices
+            if cost < best_cost:
+                best, best_cost = slices, cost
+            slices *= 2
+        return best, 16
 
 
 class _CapturedDecode:
