@@ -38,7 +38,7 @@ class _Context(StepContext):
         wanted = (512 + blocks - 1) // blocks
         return max(1, min(wanted, pages, 32))
 
-    def decode_plan(self, n_kv_heads: int):
+    def decode_plan(self, n_kv_heads: int, group: int = 1):
         """(slices, waves per block) for the matrix-core decode kernel.  Up to 256 (sequence,
         kv head) pairs: blocks of 16 waves, a tile of 16 keys per wave at a time, and as many
         slices of the key range as shorten a wave's walk by more than the merge kernel costs,
@@ -47,7 +47,9 @@ class _Context(StepContext):
         0.1 us for each slice it reads.  More pairs than that: blocks of 4 waves, see
         `decode_splits`."""
         context = self._fixed_context or self.max_context
-        pairs = self.n_seqs * n_kv_heads
+        # (a block of 16 waves takes at most 4 query heads of a group: larger groups have
+        # several blocks per pair)
+        pairs = self.n_seqs * n_kv_heads * ((group + 3) // 4)
         if pairs > 256:
             return self.decode_splits(n_kv_heads), 4
         tiles = (context + 15) // 16

@@ -113,7 +113,7 @@ class Attention:
         out = ctx.buffer("attn.out", (n, spec.q_width))
         part_o = part_ml = None
         if ctx.decode:
-            splits, waves = (ctx.decode_plan(spec.n_kv_heads) if self.matrix_cores
+            splits, waves = (ctx.decode_plan(spec.n_kv_heads, self.group) if self.matrix_cores
                              else (ctx.decode_splits(spec.n_kv_heads), 4))
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
