@@ -9,6 +9,7 @@ session as it was; the reference holds the same contract, runtime/src/qwen3.cpp:
 """
 from __future__ import annotations
 
+import numbers
 import os
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -233,10 +234,12 @@ class Session:
             tokens = list(tokens)
             if not tokens:
                 raise ValueError("an entry brings at least one token")
-            for token in tokens:
-                if not isinstance(token, int) or isinstance(token, bool) \
-                        or not 0 <= token < vocab:
+            for index, token in enumerate(tokens):
+                if not isinstance(token, numbers.Integral) or isinstance(token, bool):
+                    raise ValueError(f"token ids are integers, got {token!r}")
+                if not 0 <= token < vocab:
                     raise ValueError(f"token id {token!r} is outside the vocabulary of {vocab}")
+                tokens[index] = int(token)
             want = list(want)
             for w in want:
                 if not 0 <= w < len(tokens):

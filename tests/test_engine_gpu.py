@@ -259,9 +259,17 @@ def test_refused_steps_change_nothing(models):
     session.step([(slot, [1, 2, 3], [2])])
     before = session.cache.kv_k[0].clone()
     for entries in ([(slot, [256], [0])], [(slot, [-1], [0])], [(slot, [], [])],
-                    [(slot, [1], [1])], [(5, [1], [0])], [(slot, [1], [0]), (slot, [2], [0])]):
+                    [(slot, [1], [1])], [(5, [1], [0])], [(slot, [1], [0]), (slot, [2], [0])],
+                    [(slot, [1.0], [0])], [(slot, [True], [0])]):
         with pytest.raises(ValueError):
             session.step(entries)
+    import numpy as np
+    again = session.step([(slot, [np.int64(7), np.int32(9)], [1])])     # integers of any kind
+    assert again.shape == (1, 256) and session.length(slot) == 5
+    session.end(slot)
+    slot = session.begin()
+    session.step([(slot, [1, 2, 3], [2])])
+    before = session.cache.kv_k[0].clone()
     with pytest.raises(CacheFull):
         session.step([(slot, [1] * 126, [])])          # 3 + 126 > 128 positions of the model
     other = session.begin()
