@@ -7,7 +7,8 @@ Prints one JSON line.  `value` is decoded tokens per second at the given batch a
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
 sampling, and the tokens fed back).  `prefill` is one prompt of 2,048 tokens;
 `roofline` prices the decode step against HBM bandwidth (every weight it uses once,
-plus the cache of the live requests); `points` hold decode at batch 1 and 64.
+plus the cache of the live requests); `points` hold decode at batch 1 and 64, and the
+headline batch without HIP graphs.
 `--only generate` times the generation loop instead: a batch of prompts with lengths
 uniform in [64, 2048] that start together, then `--new-tokens` greedy tokens each (the
 workload named for the 0.6B shape, with `--shape 0.6b --batch 32 --context 8192`).
@@ -72,13 +73,13 @@ def synthetic_prompts(cfg, batch, length, seed):
     return torch.randint(0, cfg.vocab_size, (batch, length), generator=g).tolist()
 
 
-def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT):
+def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True):
     """(ms per step, mean context during the timed steps)."""
     import torch
     import edge_infer_amd as ei
     from edge_infer_amd.sampling import Sampler, SamplingParams
     session = ei.Session(model, max_tokens=batch * CONTEXT, max_seqs=batch,
-                         max_seq_tokens=CONTEXT)
+                         max_seq_tokens=CONTEXT, graphs=graphs)
     sampler = Sampler(model.device)
     greedy = SamplingParams(temperature=0.0)
     prompts = synthetic_prompts(cfg, batch, prompt, seed=100 + batch)
@@ -229,6 +230,10 @@ def main():
         for name, batch in (("decode_b1", 1), ("decode_b64", 64)):
             ms, _ = measure_decode(model, cfg, batch, max(8, args.steps // 2), args.warmup)
             points[name] = round(batch * 1000.0 / ms, 1)
+        # the headline batch with every kernel launched by the host instead of from a HIP graph
+        ms, _ = measure_decode(model, cfg, args.batch, max(8, args.steps // 2), args.warmup,
+                               graphs=False)
+        points[f"decode_b{args.batch}_eager"] = round(args.batch * 1000.0 / ms, 1)
     from edge_infer_amd.csrc import lib
     record = {
         "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch} after "
