@@ -45,12 +45,16 @@ class WorkspacePlan:
             if a.name in self._index:
                 raise ValueError(f"duplicate workspace allocation: {a.name}")
             self._index[a.name] = i
-            for other in self.allocations[:i]:
-                lifetimes = a.first_use <= other.last_use and other.first_use <= a.last_use
-                storage = a.offset < other.offset + other.bytes and other.offset < a.offset + a.bytes
-                if lifetimes and storage:
+        # in order of first use only the values still live need comparing (a step of many
+        # layers has hundreds of values and a handful live at a time)
+        live: List[Allocation] = []
+        for a in sorted(self.allocations, key=lambda x: x.first_use):
+            live = [other for other in live if other.last_use >= a.first_use]
+            for other in live:
+                if a.offset < other.offset + other.bytes and other.offset < a.offset + a.bytes:
                     raise ValueError(f"overlapping live workspace allocations: {other.name} "
                                      f"and {a.name}")
+            live.append(a)
 
     def __contains__(self, name: str) -> bool:
         return name in self._index
@@ -82,9 +86,11 @@ class WorkspacePlan:
 class WorkspacePlanner:
     def __init__(self):
         self._requests: List[Allocation] = []
+        self._names = set()
 
     def clear(self) -> None:
         self._requests.clear()
+        self._names.clear()
 
     def add_request(self, name: str, nbytes: int, first_use: int, last_use: int,
                     alignment: int = 256) -> None:
@@ -96,8 +102,9 @@ class WorkspacePlanner:
             raise ValueError(f"workspace request has an invalid lifetime for {name}")
         if not _power_of_two(alignment):
             raise ValueError(f"workspace alignment must be a power of two for {name}")
-        if any(r.name == name for r in self._requests):
+        if name in self._names:
             raise ValueError(f"duplicate workspace request: {name}")
+        self._names.add(name)
         self._requests.append(Allocation(name, 0, int(nbytes), int(first_use), int(last_use),
                                          int(alignment)))
 
