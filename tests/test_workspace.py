@@ -132,3 +132,20 @@ def test_without_a_step_the_workspace_hands_out_one_buffer_per_name():
     b = ws.get("a", (4, 4), torch.float32)
     assert a.data_ptr() == b.data_ptr()
     assert ws.get("c", (3,), torch.float32).data_ptr() != a.data_ptr()
+
+
+def test_old_plans_are_dropped_and_planned_again_when_needed():
+    ws = Workspace("cpu")
+    for n in range(Workspace.MAX_PLANS + 3):
+        run_step(ws, ("shape", n))
+    assert len(ws._plans) == Workspace.MAX_PLANS and ("shape", 0) not in ws._plans
+    run_step(ws, ("shape", 0))                 # recorded anew ...
+    a, b, c, a2, d = run_step(ws, ("shape", 0))
+    assert c.data_ptr() == a.data_ptr()        # ... and planned again
+    # a step that fails in the middle leaves nothing behind
+    ws.start("broken")
+    ws.get("a", (10,), torch.float32)
+    ws.abort()
+    assert "broken" not in ws._plans
+    run_step(ws, "broken")
+    assert "broken" in ws._plans
