@@ -10,7 +10,7 @@
 // o = sum w_t v_t / sum w_t; query head h reads kv head h / (nq / nkv).
 // operators/src/cuda/execution.cu:137-179, runtime/src/qwen.cpp:374-402,
 // split merge: operators/src/cuda/kernels/gather_fa_variable.cu:14-118.
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

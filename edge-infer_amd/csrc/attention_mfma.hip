@@ -14,7 +14,7 @@
 // t <= p (and t > p - window), scale 1/sqrt(d) or the given one, float32 softmax.
 #include <type_traits>
 
-#include "common.cuh"
+#include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));

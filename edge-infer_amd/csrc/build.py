@@ -65,7 +65,7 @@ def _hipcc() -> str:
 def _stamp(name: str) -> str:
     digest = hashlib.sha256()
     digest.update((SOURCE_DIR / f"{name}.hip").read_bytes())
-    for header in sorted(SOURCE_DIR.glob("*.cuh")):
+    for header in sorted(SOURCE_DIR.glob("*.h")):
         digest.update(header.read_bytes())
     digest.update(" ".join(FLAGS).encode())
     return digest.hexdigest()

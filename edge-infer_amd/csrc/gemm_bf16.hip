@@ -17,7 +17,7 @@
 // Accumulation is float32 throughout, as in the reference's cublasGemmEx call
 // (operators/src/cuda/execution.cu:319-323); the sums stay float32 and the consumer rounds
 // once when it stores in the storage type.
-#include "common.cuh"
+#include "common.h"
 
 #include <type_traits>
 

@@ -8,7 +8,7 @@
 // kernels below computed it: two tiled ones (64 x 64 outputs a block; 128 x 128 for many rows
 // with K in fours) and the weight-streaming one for up to 8 rows (decode), which reads every
 // weight row in kilobyte pieces.
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

@@ -10,7 +10,7 @@
 // runtime/include/execution/decoder.hpp:125-140; rotate-half pairs (i, i + d/2),
 // x' = x cos - y sin, y' = x sin + y cos, operators/src/cuda/execution.cu:79-122;
 // keys stored after norm and rotation, values raw, decoder.hpp:137-140.
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

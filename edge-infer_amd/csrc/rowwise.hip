@@ -6,7 +6,7 @@
 // Formulas: operators/src/cuda/execution.cu:67-78 (gather),
 // operators/src/cuda/rms_norm_cuda.cu:19-101 (x * rsqrt(mean(x^2) + eps) * w),
 // operators/src/cuda/silu_cuda.cu:44-56 (silu(gate) * up) of the reference.
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 

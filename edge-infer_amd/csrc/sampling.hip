@@ -10,7 +10,7 @@
 // select and only the k candidates are sorted.  The uniform number comes from a
 // counter-based generator keyed by (seed, request stream, step counter), so a
 // request draws the same numbers alone or in any batch.
-#include "common.cuh"
+#include "common.h"
 
 namespace {
 
