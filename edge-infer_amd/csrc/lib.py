@@ -75,6 +75,7 @@ _SIGNATURES = {
     "sampling": {
         "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
         "ei_argmax_partial_size": [c_int, c_int],
+        "ei_argmax_static": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
         "ei_sample": [c_void_p, c_int, c_int, c_float, c_float, c_int, c_ulonglong, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
         "ei_sample_scratch_size": [c_int, c_int],
@@ -450,6 +451,25 @@ def argmax(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None, parti
                            None if partial is None else _gpu(partial, "partial", torch.float32),
                            0 if partial is None else partial.numel() // 2, _stream())
     _check(lib, status, "argmax")
+
+
+ARGMAX_STATIC_MAX_PARTIALS = 65536
+
+
+def argmax_static(logits: torch.Tensor, tokens: torch.Tensor, probabilities=None) -> None:
+    """`argmax` without a buffer from the caller and without any allocation: the partial results
+    of a wide vocabulary live in a device array of the library (at most 65536 pairs of row and
+    chunk of 4096 logits; larger requests are refused).  Calls that overlap on one GPU race."""
+    lib = library("sampling")
+    rows, vocab = logits.shape
+    if tokens.numel() < rows:
+        raise KernelError("argmax_static: tokens shorter than the rows")
+    status = lib.ei_argmax_static(_gpu(logits, "logits", torch.float32), rows, vocab,
+                                  _gpu(tokens, "tokens", torch.int32),
+                                  None if probabilities is None
+                                  else _gpu(probabilities, "probabilities", torch.float32),
+                                  _stream())
+    _check(lib, status, "argmax_static")
 
 
 def sample_scratch_size(rows: int, vocab: int) -> int:

@@ -11,6 +11,9 @@
 // counter-based generator keyed by (seed, request stream, step counter), so a
 // request draws the same numbers alone or in any batch.
 #include "common.h"
+#include "sampling_static.h"
+
+#include <atomic>
 
 namespace {
 
@@ -523,6 +526,54 @@ extern "C" int ei_argmax(const float* logits, int rows, int V, int32_t* tokens,
     EI_LAUNCH_CHECK();
   }
   argmax_kernel<<<rows, kThreads, 0, stream>>>(logits, V, tokens, probabilities);
+  EI_LAUNCH_CHECK();
+}
+
+// The partial results of ei_argmax_static: one copy on every GPU, at an address of its own
+// there.  Host code never passes this name to a kernel (on the host it is a stand-in, not a
+// device address); it asks the runtime for the address once per device and uses that.
+static __device__ __align__(256) float2 argmax_static_scratch[EI_ARGMAX_STATIC_MAX_PARTIALS];
+
+constexpr int kStaticDevices = 64;
+static std::atomic<float2*> argmax_static_address[kStaticDevices];
+
+// See sampling_static.h.  The first call on a device looks the array's address up (with that
+// device current) and keeps it; nothing is allocated then or later.
+extern "C" int ei_argmax_static(const float* logits, int rows, int V, int32_t* tokens,
+                                float* probabilities, hipStream_t stream) {
+  EI_REQUIRE(rows > 0 && V > 0, "argmax_static: sizes must be positive");
+  EI_REQUIRE(logits && tokens, "argmax_static: null pointer");
+  const long long chunks = (static_cast<long long>(V) + kArgmaxChunk - 1) / kArgmaxChunk;
+  if (V <= 2 * kArgmaxChunk) {          // one block a row: no partial results
+    argmax_kernel<<<rows, kThreads, 0, stream>>>(logits, V, tokens, probabilities);
+    EI_LAUNCH_CHECK();
+  }
+  EI_REQUIRE(static_cast<long long>(rows) * chunks <= EI_ARGMAX_STATIC_MAX_PARTIALS,
+             "argmax_static: rows * ceil(V / 4096) exceeds the 65536 partial results that the "
+             "library's static buffer holds");
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) {
+    ei_set_error(hipGetErrorString(status));
+    return static_cast<int>(status);
+  }
+  EI_REQUIRE(device >= 0 && device < kStaticDevices, "argmax_static: device index out of range");
+  float2* partial = argmax_static_address[device].load(std::memory_order_acquire);
+  if (partial == nullptr) {
+    void* address = nullptr;
+    status = hipGetSymbolAddress(&address, HIP_SYMBOL(argmax_static_scratch));
+    if (status != hipSuccess) {
+      ei_set_error(hipGetErrorString(status));
+      return static_cast<int>(status);
+    }
+    EI_REQUIRE(address != nullptr, "argmax_static: the static buffer has no device address");
+    partial = static_cast<float2*>(address);
+    argmax_static_address[device].store(partial, std::memory_order_release);
+  }
+  argmax_chunks_kernel<<<dim3(static_cast<unsigned>(chunks), rows), kArgmaxThreads, 0, stream>>>(
+      logits, V, partial);
+  argmax_merge_kernel<<<rows, EI_WAVE, 0, stream>>>(partial, static_cast<int>(chunks), tokens,
+                                                    probabilities);
   EI_LAUNCH_CHECK();
 }
 
