@@ -3,9 +3,10 @@
 Tensors keep the precision they are stored in when that is bfloat16 or 32-bit
 float; 16-bit IEEE floats become bfloat16, 64-bit floats become 32-bit, and
 integer tables become int32.  The parts decide later what they compute in.
-File handling follows frontend/checkpoint.py:58-105 of the reference: a single
-`model.safetensors` or a `model.safetensors.index.json` whose shards must stay
-inside the model folder; nothing is ever downloaded.
+A folder holds a single `model.safetensors` or a `model.safetensors.index.json` over
+several files, which must lie inside the folder; nothing is ever downloaded (the same
+rules as the reference's loader, frontend/checkpoint.py:58-105).  The container is read by
+this package itself (`safetensors_file.py`): memory-mapped, tensor by tensor.
 """
 from __future__ import annotations
 
@@ -54,59 +55,75 @@ class WeightsError(ValueError):
         return "\n".join(lines)
 
 
-def _shard_path(root: Path, name) -> Path:
-    if not isinstance(name, str) or not name or Path(name).is_absolute():
-        raise ValueError("checkpoint shard names must be relative paths")
-    path = (root / name).resolve()
-    try:
-        path.relative_to(root)
-    except ValueError as error:
-        raise ValueError("checkpoint shards must stay inside the model folder") from error
-    if not path.is_file():
-        raise FileNotFoundError(path)
-    return path
+INDEX_FILE = "model.safetensors.index.json"
+SINGLE_FILE = "model.safetensors"
 
 
-def _stored_precision(tensor: torch.Tensor) -> torch.Tensor:
+def kept_precision(tensor: torch.Tensor) -> torch.Tensor:
+    """bfloat16, float32 and int32 stay as they are; float16 becomes bfloat16, float64
+    float32, every other integer type int32."""
     if tensor.dtype in (torch.bfloat16, torch.float32, torch.int32):
         return tensor
-    if tensor.dtype == torch.float16:
-        return tensor.to(torch.bfloat16)
     if tensor.dtype == torch.float64:
         return tensor.to(torch.float32)
-    if not tensor.dtype.is_floating_point:
-        return tensor.to(torch.int32)
-    return tensor.to(torch.bfloat16)
+    if tensor.dtype.is_floating_point:
+        return tensor.to(torch.bfloat16)
+    return tensor.to(torch.int32)
+
+
+def _file_inside(folder: Path, relative) -> Path:
+    """The file `relative` names, which must lie inside `folder` (an index is data from
+    outside: it must not be able to point anywhere else on the machine)."""
+    if not isinstance(relative, str) or relative == "" or Path(relative).is_absolute():
+        raise ValueError(f"a checkpoint file is named by a path relative to the model folder, "
+                         f"got {relative!r}")
+    target = (folder / relative).resolve()
+    if folder not in target.parents:
+        raise ValueError(f"every checkpoint file must lie inside the model folder; "
+                         f"'{relative}' does not")
+    if not target.is_file():
+        raise FileNotFoundError(target)
+    return target
+
+
+def checkpoint_files(model_dir) -> Dict[Path, Optional[List[str]]]:
+    """file -> the tensor names to take from it (None: all it holds).  A folder holds either
+    an index over several files or the one file `model.safetensors`."""
+    folder = Path(model_dir).resolve()
+    index_path = folder / INDEX_FILE
+    if not index_path.is_file():
+        return {_file_inside(folder, SINGLE_FILE): None}
+    listing = json.loads(index_path.read_text(encoding="utf-8"))
+    placement = listing.get("weight_map") if isinstance(listing, dict) else None
+    if not isinstance(placement, dict) or not placement:
+        raise ValueError(f"{index_path} must hold a 'weight_map' from tensor names to files")
+    files: Dict[Path, Optional[List[str]]] = {}
+    for tensor_name, file_name in placement.items():
+        files.setdefault(_file_inside(folder, file_name), []).append(tensor_name)
+    return files
 
 
 def read_tensors(model_dir) -> Dict[str, torch.Tensor]:
-    """Every tensor of the folder's safetensors file(s), on the host."""
-    from safetensors import safe_open
+    """name -> tensor for everything the folder's checkpoint holds, in the kept precision.
+    The tensors are views of the memory-mapped files (see `SafetensorsFile`) unless their
+    type had to be converted, so asking for all of them reads next to nothing; nothing is
+    ever downloaded.  EDGE_INFER_VERBOSE_WEIGHTS=1 lists them on standard output."""
+    from .safetensors_file import SafetensorsFile
 
-    root = Path(model_dir).resolve()
-    index_path = root / "model.safetensors.index.json"
-    if index_path.is_file():
-        with index_path.open(encoding="utf-8") as source:
-            index = json.load(source)
-        weight_map = index.get("weight_map") if isinstance(index, dict) else None
-        if not isinstance(weight_map, dict) or not weight_map:
-            raise ValueError("the safetensors index must hold a nonempty weight_map")
-        shards: Dict[Path, Optional[List[str]]] = {}
-        for name, shard in weight_map.items():
-            shards.setdefault(_shard_path(root, shard), []).append(name)
-    else:
-        shards = {_shard_path(root, "model.safetensors"): None}
-    # EDGE_INFER_VERBOSE_WEIGHTS=1 lists what is read, as in frontend/checkpoint.py:88-99
-    verbose = os.environ.get("EDGE_INFER_VERBOSE_WEIGHTS") == "1"
+    chatty = os.environ.get("EDGE_INFER_VERBOSE_WEIGHTS") == "1"
     tensors: Dict[str, torch.Tensor] = {}
-    for path, names in shards.items():
-        with safe_open(str(path), framework="pt", device="cpu") as source:
-            for name in (source.keys() if names is None else names):
-                tensors[name] = _stored_precision(source.get_tensor(name))
-                if verbose:
-                    print(f"Loaded {name}: {tuple(tensors[name].shape)}, {tensors[name].dtype}")
+    for path, wanted in checkpoint_files(model_dir).items():
+        container = SafetensorsFile(path)
+        for name in (list(container.names()) if wanted is None else wanted):
+            if name not in container:
+                raise ValueError(f"the index places '{name}' in {path.name}, which does not "
+                                 f"hold it")
+            tensors[name] = kept_precision(container.tensor(name))
+            if chatty:
+                print(f"{path.name}: {name} {list(tensors[name].shape)} "
+                      f"{str(tensors[name].dtype).replace('torch.', '')}")
     if not tensors:
-        raise ValueError("the checkpoint holds no tensors")
+        raise ValueError(f"the checkpoint in {model_dir} holds no tensors")
     return tensors
 
 

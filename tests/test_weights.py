@@ -116,6 +116,59 @@ def test_sharded_checkpoint_and_path_containment(tmp_path):
         read_tensors(tmp_path)
 
 
+def test_the_container_is_read_by_this_package_and_refuses_what_does_not_add_up(tmp_path):
+    """The reader agrees with the library that wrote the file, gives views of the mapping
+    (no bytes read until touched) and refuses headers that lie."""
+    import struct
+    from edge_infer_amd.weights.safetensors_file import SafetensorsFile
+    tensors = {"m": torch.arange(12, dtype=torch.float32).reshape(3, 4),
+               "h": torch.randn(5, 2).to(torch.float16), "empty": torch.zeros(0, 7),
+               "flags": torch.tensor([True, False, True]), "bytes": torch.arange(5, dtype=torch.uint8)}
+    path = tmp_path / "model.safetensors"
+    save_file(tensors, str(path), metadata={"format": "pt"})
+    container = SafetensorsFile(path)
+    assert sorted(container.names()) == sorted(tensors) and container.metadata == {"format": "pt"}
+    for name, tensor in tensors.items():
+        assert container.shape(name) == tuple(tensor.shape) and container.dtype(name) == tensor.dtype
+        assert torch.equal(container.tensor(name), tensor)
+    loaded = read_tensors(tmp_path)
+    assert loaded["flags"].dtype == torch.int32 and loaded["flags"].tolist() == [1, 0, 1]
+    assert loaded["bytes"].dtype == torch.int32 and loaded["h"].dtype == torch.bfloat16
+    # a view, not a copy: two reads of a tensor share their bytes; writing to it changes no file
+    view = container.tensor("m")
+    assert view.data_ptr() == container.tensor("m").data_ptr()
+    view.fill_(7.0)
+    assert torch.equal(SafetensorsFile(path).tensor("m"), tensors["m"])
+    raw = path.read_bytes()
+    (length,) = struct.unpack("<Q", raw[:8])
+    header = json.loads(raw[8:8 + length])
+
+    def rewritten(change):
+        changed = json.loads(json.dumps(header))
+        change(changed)
+        text = json.dumps(changed).encode()
+        (tmp_path / "bad.safetensors").write_bytes(struct.pack("<Q", len(text)) + text
+                                                    + raw[8 + length:])
+        return tmp_path / "bad.safetensors"
+    with pytest.raises(ValueError, match="does not fit"):
+        SafetensorsFile(rewritten(lambda h: h["m"].update(shape=[3, 5])))
+    with pytest.raises(ValueError, match="does not fit"):
+        SafetensorsFile(rewritten(lambda h: h["m"].update(data_offsets=[0, 10 ** 9])))
+    with pytest.raises(ValueError, match="unsupported"):
+        SafetensorsFile(rewritten(lambda h: h["m"].update(dtype="F8_E4M3")))
+    (tmp_path / "bad.safetensors").write_bytes(struct.pack("<Q", 10 ** 12) + b"{}")
+    with pytest.raises(ValueError, match="header claims"):
+        SafetensorsFile(tmp_path / "bad.safetensors")
+    (tmp_path / "bad.safetensors").write_bytes(b"abc")
+    with pytest.raises(ValueError, match="too short"):
+        SafetensorsFile(tmp_path / "bad.safetensors")
+    # an index that names a tensor its file does not hold
+    (tmp_path / "model.safetensors.index.json").write_text(
+        json.dumps({"weight_map": {"nowhere": "model.safetensors"}}))
+    with pytest.raises(ValueError, match="hold it"):
+        read_tensors(tmp_path)
+
+
 def test_parameter_inventory_matches_the_architecture():
     cfg = tiny_config("B")
     every = model_parameters(cfg.model_spec())
@@ -131,8 +184,9 @@ def test_parameter_inventory_matches_the_architecture():
 
 
 def test_verbose_listing_of_what_is_read(tmp_path, monkeypatch, capsys):
-    """EDGE_INFER_VERBOSE_WEIGHTS=1 lists every tensor as the reference's loader does
-    (frontend/checkpoint.py:88-99); without it nothing is printed."""
+    """EDGE_INFER_VERBOSE_WEIGHTS=1 lists every tensor with its file, shape and type (the
+    reference's loader has such a listing too, frontend/checkpoint.py:88-99); without it
+    nothing is printed."""
     folder = make_folder("A", tmp_path)
     read_tensors(folder)
     assert capsys.readouterr().out == ""
@@ -140,7 +194,7 @@ def test_verbose_listing_of_what_is_read(tmp_path, monkeypatch, capsys):
     tensors = read_tensors(folder)
     lines = capsys.readouterr().out.strip().split("\n")
     assert len(lines) == len(tensors)
-    assert any(line.startswith("Loaded model.embed_tokens.weight: (256, 64)") for line in lines)
+    assert "model.safetensors: model.embed_tokens.weight [256, 64] bfloat16" in lines
 
 
 def test_optional_biases_are_taken_when_the_checkpoint_holds_them(tmp_path):
