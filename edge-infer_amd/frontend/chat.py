@@ -49,20 +49,95 @@ def render_chat(messages, model_path) -> str:
     return text + "<|im_start|>assistant\n"
 
 
-def decode_stream_incremental(tokenizer, token_ids, rendered_text):
-    """(new text that is safe to print, text rendered so far): text that ends inside a
-    multi-byte character is held back until the character is complete."""
-    decoded = tokenizer.decode(token_ids, skip_special_tokens=True)
-    prefix = 0
-    limit = min(len(rendered_text), len(decoded))
-    while prefix < limit and rendered_text[prefix] == decoded[prefix]:
-        prefix += 1
-    pending = decoded[prefix:]
-    broken = pending.find("�")
-    if broken != -1:
-        safe = pending[:broken]
-        return safe, decoded[:prefix + len(safe)]
-    return pending, decoded
+def _byte_alphabet():
+    """The printable stand-in of every byte in byte-level vocabularies: bytes that print
+    (33-126, 161-172, 174-255) stand for themselves, the others are numbered from 256 on in
+    ascending order.  Returns stand-in character -> byte."""
+    printable = [*range(33, 127), *range(161, 173), *range(174, 256)]
+    table, extra = {}, 0
+    for byte in range(256):
+        if byte in printable:
+            table[chr(byte)] = byte
+        else:
+            table[chr(256 + extra)] = byte
+            extra += 1
+    return table
+
+
+def _whole_characters(data) -> int:
+    """How many leading bytes of `data` can be decoded without cutting a UTF-8 character:
+    if a lead byte among the last three announces more bytes than have arrived, the count
+    stops before it."""
+    size = len(data)
+    for back in range(1, min(4, size) + 1):
+        byte = data[size - back]
+        if byte & 0xC0 == 0x80:
+            continue                          # a continuation byte: look further back
+        expected = 1 if byte < 0xC0 else 2 if byte < 0xE0 else 3 if byte < 0xF0 else 4
+        return size if back >= expected else size - back
+    return size
+
+
+class TextStream:
+    """Turns generated token ids into printable text piece by piece.
+
+    Tokens of a byte-level vocabulary (the kind Qwen checkpoints have) are byte strings and
+    a character may be spread over several tokens: their bytes are collected, and only the
+    bytes that form whole characters are decoded and handed out; an unfinished tail waits for
+    the next token.  For any other tokenizer the whole answer is decoded again at every token
+    and what is new is handed out, except a tail of replacement characters, which the decoder
+    writes for a character it cannot finish yet."""
+
+    def __init__(self, tokenizer):
+        self.tokenizer = tokenizer
+        self.text = ""                      # everything handed out so far
+        self._bytes = bytearray()           # byte-level: bytes not handed out yet
+        self._ids = []                      # otherwise: every token so far
+        self._alphabet = self._special = None
+        describe = getattr(tokenizer, "to_str", None)
+        if describe is not None:
+            decoder = json.loads(describe()).get("decoder") or {}
+            stages = decoder.get("decoders", [decoder])
+            if any(stage.get("type") == "ByteLevel" for stage in stages):
+                self._alphabet = _byte_alphabet()
+                self._special = {index: token.content for index, token
+                                 in tokenizer.get_added_tokens_decoder().items()}
+
+    def push(self, token: int) -> str:
+        """The text that this token completes (possibly empty)."""
+        if self._alphabet is None:
+            self._ids.append(token)
+            decoded = self.tokenizer.decode(self._ids, skip_special_tokens=True)
+            settled = decoded.rstrip("\ufffd")
+            if len(decoded) - len(settled) > 3:      # more than one character can lack: real ones
+                settled = decoded
+            if not settled.startswith(self.text):    # the decoder changed its mind: keep what is out
+                return ""
+            piece = settled[len(self.text):]
+        else:
+            if token in self._special:
+                return ""                            # markers of the chat layout are not text
+            symbol = self.tokenizer.id_to_token(token) or ""
+            try:
+                self._bytes += bytes(self._alphabet[char] for char in symbol)
+            except KeyError:                         # an added plain-text token
+                self._bytes += symbol.encode("utf-8")
+            whole = _whole_characters(self._bytes)
+            piece = bytes(self._bytes[:whole]).decode("utf-8", errors="replace")
+            del self._bytes[:whole]
+        self.text += piece
+        return piece
+
+    def finish(self) -> str:
+        """What was still held back when generation ended."""
+        if self._alphabet is None:
+            decoded = self.tokenizer.decode(self._ids, skip_special_tokens=True) if self._ids else ""
+            piece = decoded[len(self.text):] if decoded.startswith(self.text) else ""
+        else:
+            piece = bytes(self._bytes).decode("utf-8", errors="replace")
+            self._bytes.clear()
+        self.text += piece
+        return piece
 
 
 def build_parser() -> argparse.ArgumentParser:
@@ -93,27 +168,26 @@ def build_parser() -> argparse.ArgumentParser:
 def generate_once(session, input_ids, args, tokenizer, out=sys.stdout):
     """Stream one answer; returns (token ids, seconds from the first token, text)."""
     max_length = min(session.capacity, len(input_ids) + args.max_new_tokens)
-    tokens, rendered, started = [], "", [None]
+    tokens, started = [], [None]
+    stream = TextStream(tokenizer) if tokenizer is not None else None
 
     def on_token(token):
         if started[0] is None:
             started[0] = time.monotonic()
         tokens.append(token)
-        if tokenizer is None:
-            print(token, end=" ", file=out, flush=True)
-            return
-        nonlocal rendered
-        piece, rendered = decode_stream_incremental(tokenizer, tokens, rendered)
+        piece = f"{token} " if stream is None else stream.push(token)
         if piece:
             print(piece, end="", file=out, flush=True)
 
     session.generate(input_ids, on_token, max_length=max_length, temperature=args.temperature,
                      top_p=args.top_p, top_k=args.top_k)
     elapsed = time.monotonic() - started[0] if started[0] is not None else 0.0
-    text = tokenizer.decode(tokens, skip_special_tokens=True) if tokenizer is not None else ""
-    if tokenizer is not None and text[len(rendered):]:
-        print(text[len(rendered):], end="", file=out, flush=True)
-    return tokens, elapsed, text
+    if stream is None:
+        return tokens, elapsed, ""
+    rest = stream.finish()
+    if rest:
+        print(rest, end="", file=out, flush=True)
+    return tokens, elapsed, stream.text
 
 
 def report(tokens, elapsed, out=sys.stdout):

@@ -36,17 +36,41 @@ def test_chat_rendering(tmp_path):
 
 def test_streaming_holds_back_incomplete_characters():
     class Bytes:
-        """Tokens are single bytes of UTF-8 text."""
+        """Tokens are single bytes of UTF-8 text; no description, so the stream decodes the
+        whole answer again at every token."""
         def decode(self, ids, skip_special_tokens=True):
             return bytes(ids).decode("utf-8", errors="replace")
-    tok = Bytes()
-    data = list("a€b".encode("utf-8"))          # 'a', three bytes of the euro sign, 'b'
-    shown, rendered = "", ""
-    for n in range(1, len(data) + 1):
-        piece, rendered = chat.decode_stream_incremental(tok, data[:n], rendered)
-        assert "�" not in piece
+    stream = chat.TextStream(Bytes())
+    shown = ""
+    for byte in "a\u20acb\U0001f600".encode("utf-8"):   # 1, 3, 1 and 4 bytes
+        piece = stream.push(byte)
+        assert "\ufffd" not in piece
         shown += piece
-    assert shown == "a€b"
+    assert shown + stream.finish() == "a\u20acb\U0001f600" == stream.text
+    # an answer that ends inside a character: the end hands out what there is
+    stream = chat.TextStream(Bytes())
+    assert stream.push(0x61) == "a" and stream.push(0xE2) == "" and stream.finish() == "\ufffd"
+
+
+def test_streaming_of_a_byte_level_vocabulary_collects_bytes():
+    """Characters spread over several tokens come out once complete, special tokens are
+    not text, and what a cut-off answer leaves is handed out at the end."""
+    from tokenizers import Tokenizer, decoders, models
+    alphabet = {byte: char for char, byte in chat._byte_alphabet().items()}
+    assert len(alphabet) == 256 and alphabet[ord("A")] == "A" and alphabet[0x20] == "\u0120"
+    vocab = {char: index for index, char in enumerate(alphabet[b] for b in range(256))}
+    vocab[alphabet[0xE2] + alphabet[0x82]] = 256            # two of the euro sign's three bytes
+    tokenizer = Tokenizer(models.BPE(vocab=vocab, merges=[]))
+    tokenizer.decoder = decoders.ByteLevel()
+    tokenizer.add_special_tokens(["<|im_end|>"])
+    end = tokenizer.token_to_id("<|im_end|>")
+    stream = chat.TextStream(tokenizer)
+    pieces = [stream.push(t) for t in (ord("h"), 0x20, 256, 0xAC, 0xF0, 0x9F, end, 0x98, 0x80)]
+    assert pieces == ["h", " ", "", "\u20ac", "", "", "", "", "\U0001f600"]
+    assert stream.finish() == "" and stream.text == "h \u20ac\U0001f600"
+    assert [chat._whole_characters(data) for data in
+            (b"", b"ab", b"a\xe2", b"a\xe2\x82", b"a\xe2\x82\xac", b"\xf0\x9f\x98", b"\x80\x80")] \
+        == [0, 2, 1, 1, 4, 0, 2]
 
 
 def make_word_tokenizer(folder, vocab_size):
