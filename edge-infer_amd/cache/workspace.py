@@ -1,133 +1,146 @@
-"""Offline planning of a step's workspace: values whose lifetimes do not overlap share
-storage.
+"""Laying out the buffers of a step in one arena: buffers that are never live at the same
+time share bytes.
 
-A request names a value, its size in bytes and the first and last step at which it is
-used; the planner sorts requests by (first use, last use, name) and gives each the
-smallest slot that is dead (its last value's last use lies strictly before the new
-first use), large enough and aligned, or appends a new slot.  It allocates nothing: a
-plan is a table of offsets into one arena.  Behaviour and checks follow the reference's
-planner, core/include/execution/workspace_plan.hpp:138-252 (plan validation :32-60,
-metrics :75-118).
+A step is a sequence of ticks.  Each buffer has a `Lifetime`: the tick at which it is first
+written (`born`) and the last tick at which it is read (`dies`).  `lay_out` walks the
+lifetimes in birth order and keeps a list of regions of the arena; a buffer moves into the
+tightest region whose previous tenant is dead (died strictly before the newcomer is born:
+at the same tick a kernel may still read the one while it writes the other), that is large
+enough and suitably aligned; if there is none the arena grows by a new region.  Nothing is
+allocated here: the result says where in an arena of `arena_bytes` each buffer lies.
+
+The reference plans its decoder buffers offline in the same way and this module answers
+its planner's test vectors the same way (core/include/execution/workspace_plan.hpp:138-252,
+operators/tests/decode_workspace_plan_test.cpp:16-60); the lifetimes here are not declared
+by hand but recorded from a step that ran (`parts.base.Workspace`).
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional
+from typing import Dict, Iterable, List
+
+DEFAULT_ALIGNMENT = 256
 
 
 @dataclass(frozen=True)
-class Allocation:
+class Lifetime:
+    """A buffer's need: `nbytes` from tick `born` through tick `dies`, at an address that is
+    a multiple of `alignment` (a power of two)."""
     name: str
+    nbytes: int
+    born: int
+    dies: int
+    alignment: int = DEFAULT_ALIGNMENT
+
+    def check(self) -> None:
+        if not self.name:
+            raise ValueError("a buffer needs a name")
+        if self.nbytes <= 0:
+            raise ValueError(f"buffer '{self.name}': its size must be positive")
+        if self.born > self.dies:
+            raise ValueError(f"buffer '{self.name}': it dies before it is born")
+        if self.alignment <= 0 or self.alignment & (self.alignment - 1):
+            raise ValueError(f"buffer '{self.name}': the alignment must be a power of two")
+
+
+@dataclass(frozen=True)
+class Placement:
+    """Where a buffer lies in the arena."""
+    need: Lifetime
     offset: int
-    bytes: int
-    first_use: int
-    last_use: int
-    alignment: int = 256
+
+    @property
+    def end(self) -> int:
+        return self.offset + self.need.nbytes
 
 
-def _power_of_two(value: int) -> bool:
-    return value > 0 and value & (value - 1) == 0
+class ArenaLayout:
+    """Placements by buffer name.  Construction proves the layout: every buffer inside the
+    arena and aligned, and no two buffers that are live at the same tick on the same bytes."""
 
-
-class WorkspacePlan:
-    """Offsets of named values in an arena of `total_bytes`; construction checks that
-    no two values that are live at the same time overlap in storage."""
-
-    def __init__(self, allocations: List[Allocation], total_bytes: int):
-        self.allocations = list(allocations)
-        self.total_bytes = int(total_bytes)
-        self._index: Dict[str, int] = {}
-        for i, a in enumerate(self.allocations):
-            if (not a.name or a.bytes <= 0 or a.first_use > a.last_use
-                    or not _power_of_two(a.alignment) or a.offset % a.alignment
-                    or a.offset < 0 or a.offset + a.bytes > self.total_bytes):
-                raise ValueError(f"invalid workspace allocation: {a.name}")
-            if a.name in self._index:
-                raise ValueError(f"duplicate workspace allocation: {a.name}")
-            self._index[a.name] = i
-        # in order of first use only the values still live need comparing (a step of many
-        # layers has hundreds of values and a handful live at a time)
-        live: List[Allocation] = []
-        for a in sorted(self.allocations, key=lambda x: x.first_use):
-            live = [other for other in live if other.last_use >= a.first_use]
-            for other in live:
-                if a.offset < other.offset + other.bytes and other.offset < a.offset + a.bytes:
-                    raise ValueError(f"overlapping live workspace allocations: {other.name} "
-                                     f"and {a.name}")
-            live.append(a)
+    def __init__(self, placements: Iterable[Placement], arena_bytes: int):
+        self.arena_bytes = int(arena_bytes)
+        self._by_name: Dict[str, Placement] = {}
+        for placement in placements:
+            need = placement.need
+            need.check()
+            if need.name in self._by_name:
+                raise ValueError(f"buffer '{need.name}' is placed twice")
+            if placement.offset < 0 or placement.end > self.arena_bytes:
+                raise ValueError(f"buffer '{need.name}' lies outside the arena")
+            if placement.offset % need.alignment:
+                raise ValueError(f"buffer '{need.name}' is misaligned")
+            self._by_name[need.name] = placement
+        # sweep in birth order; only buffers that have not died yet can collide
+        living: List[Placement] = []
+        for placement in sorted(self._by_name.values(), key=lambda p: p.need.born):
+            living = [other for other in living if other.need.dies >= placement.need.born]
+            for other in living:
+                if placement.offset < other.end and other.offset < placement.end:
+                    raise ValueError(f"buffers '{other.need.name}' and '{placement.need.name}' "
+                                     f"are live together on the same bytes")
+            living.append(placement)
 
     def __contains__(self, name: str) -> bool:
-        return name in self._index
+        return name in self._by_name
 
-    def at(self, name: str) -> Allocation:
+    def __len__(self) -> int:
+        return len(self._by_name)
+
+    def names(self):
+        return list(self._by_name)
+
+    def offset(self, name: str) -> int:
         try:
-            return self.allocations[self._index[name]]
+            return self._by_name[name].offset
         except KeyError:
-            raise KeyError(f"workspace allocation not found: {name}") from None
+            raise KeyError(f"the layout holds no buffer '{name}'") from None
 
-    # diagnostics of a plan
-    def requested_bytes(self) -> int:
-        return sum(a.bytes for a in self.allocations)
+    # what sharing buys
+    def bytes_asked(self) -> int:
+        """The sum of the buffers' sizes."""
+        return sum(p.need.nbytes for p in self._by_name.values())
 
-    def unaliased_bytes(self) -> int:
-        """What the values would need one after the other, each aligned."""
+    def bytes_without_sharing(self) -> int:
+        """The arena that the same buffers would need side by side, each aligned."""
         total = 0
-        for a in self.allocations:
-            total += (-total) % a.alignment + a.bytes
+        for placement in self._by_name.values():
+            total += (-total) % placement.need.alignment + placement.need.nbytes
         return total
 
-    def reused_bytes(self) -> int:
-        return max(0, self.unaliased_bytes() - self.total_bytes)
+    def bytes_saved(self) -> int:
+        return max(0, self.bytes_without_sharing() - self.arena_bytes)
 
-    def slot_count(self) -> int:
-        return len({a.offset for a in self.allocations})
+    def regions(self) -> int:
+        """Distinct places in use: the fewer for the same buffers, the more sharing."""
+        return len({p.offset for p in self._by_name.values()})
 
 
-class WorkspacePlanner:
-    def __init__(self):
-        self._requests: List[Allocation] = []
-        self._names = set()
-
-    def clear(self) -> None:
-        self._requests.clear()
-        self._names.clear()
-
-    def add_request(self, name: str, nbytes: int, first_use: int, last_use: int,
-                    alignment: int = 256) -> None:
-        if not name:
-            raise ValueError("a workspace request needs a name")
-        if nbytes <= 0:
-            raise ValueError(f"workspace request bytes must be positive for {name}")
-        if first_use > last_use:
-            raise ValueError(f"workspace request has an invalid lifetime for {name}")
-        if not _power_of_two(alignment):
-            raise ValueError(f"workspace alignment must be a power of two for {name}")
-        if name in self._names:
-            raise ValueError(f"duplicate workspace request: {name}")
-        self._names.add(name)
-        self._requests.append(Allocation(name, 0, int(nbytes), int(first_use), int(last_use),
-                                         int(alignment)))
-
-    def build(self) -> WorkspacePlan:
-        ordered = sorted(self._requests, key=lambda r: (r.first_use, r.last_use, r.name))
-        slots: List[List[int]] = []          # [offset, capacity, last use]
-        allocations: List[Allocation] = []
-        total = 0
-        for request in ordered:
-            best: Optional[List[int]] = None
-            for slot in slots:
-                # a last use at the new first use still overlaps
-                if (slot[2] >= request.first_use or slot[1] < request.bytes
-                        or slot[0] % request.alignment):
-                    continue
-                if best is None or (slot[1], slot[0]) < (best[1], best[0]):
-                    best = slot
-            if best is None:
-                offset = (total + request.alignment - 1) // request.alignment * request.alignment
-                best = [offset, request.bytes, request.last_use]
-                slots.append(best)
-                total = offset + request.bytes
-            allocations.append(Allocation(request.name, best[0], request.bytes, request.first_use,
-                                          request.last_use, request.alignment))
-            best[2] = request.last_use
-        return WorkspacePlan(allocations, total)
+def lay_out(lifetimes: Iterable[Lifetime]) -> ArenaLayout:
+    needs = list(lifetimes)
+    seen = set()
+    for need in needs:
+        need.check()
+        if need.name in seen:
+            raise ValueError(f"buffer '{need.name}' is asked for twice")
+        seen.add(need.name)
+    needs.sort(key=lambda need: (need.born, need.dies, need.name))
+    regions: List[List[int]] = []          # [offset, size, tick at which its tenant dies]
+    placements: List[Placement] = []
+    arena = 0
+    for need in needs:
+        home = None
+        for region in regions:
+            offset, size, free_after = region
+            if free_after >= need.born or size < need.nbytes or offset % need.alignment:
+                continue
+            if home is None or (size, offset) < (home[1], home[0]):
+                home = region
+        if home is None:
+            offset = -(-arena // need.alignment) * need.alignment
+            home = [offset, need.nbytes, need.dies]
+            regions.append(home)
+            arena = offset + need.nbytes
+        home[2] = need.dies
+        placements.append(Placement(need, home[0]))
+    return ArenaLayout(placements, arena)

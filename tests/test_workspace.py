@@ -1,66 +1,62 @@
-"""The workspace planner (no GPU): the reference's own vectors, its refusals, and the
-record-then-plan behaviour of the step workspace on CPU tensors."""
+"""The arena layout of a step's buffers (no GPU): the reference's own vectors, what is
+refused, and the record-then-plan behaviour of the step workspace on CPU tensors."""
 import pytest
 import torch
 
-from edge_infer_amd.cache.workspace import Allocation, WorkspacePlan, WorkspacePlanner
+from edge_infer_amd.cache.workspace import ArenaLayout, Lifetime, Placement, lay_out
 from edge_infer_amd.parts.base import Workspace
 
 
 def build(*requests):
-    planner = WorkspacePlanner()
-    for request in requests:
-        planner.add_request(*request)
-    return planner.build()
+    return lay_out(Lifetime(*request) for request in requests)
 
 
 def test_reference_vectors():
     """operators/tests/decode_workspace_plan_test.cpp:16-60."""
     plan = build(("residual", 1024, 0, 2), ("attn_proj", 1024, 3, 4))
-    assert plan.total_bytes == 1024 and plan.at("residual").offset == plan.at("attn_proj").offset
+    assert plan.arena_bytes == 1024 and plan.offset("residual") == plan.offset("attn_proj")
     plan = build(("q_buf", 1024, 0, 3), ("k_buf", 1024, 2, 4))
-    assert plan.total_bytes == 2048 and plan.at("q_buf").offset != plan.at("k_buf").offset
+    assert plan.arena_bytes == 2048 and plan.offset("q_buf") != plan.offset("k_buf")
     plan = build(("small", 300, 0, 0, 256), ("aligned", 512, 1, 1, 512))
-    assert plan.at("small").offset % 256 == 0 and plan.at("aligned").offset % 512 == 0
+    assert plan.offset("small") % 256 == 0 and plan.offset("aligned") % 512 == 0
     plan = build(("large_1", 1024, 0, 0), ("small_mid", 256, 1, 1), ("large_2", 1024, 2, 2))
-    assert plan.total_bytes == 1024
-    assert plan.at("large_1").offset == plan.at("small_mid").offset == plan.at("large_2").offset
+    assert plan.arena_bytes == 1024
+    assert plan.offset("large_1") == plan.offset("small_mid") == plan.offset("large_2")
 
 
 def test_a_last_use_at_the_new_first_use_still_overlaps():
     plan = build(("a", 512, 0, 2), ("b", 512, 2, 3))
-    assert plan.at("a").offset != plan.at("b").offset
+    assert plan.offset("a") != plan.offset("b")
     plan = build(("a", 512, 0, 1), ("b", 512, 2, 3))
-    assert plan.at("a").offset == plan.at("b").offset
+    assert plan.offset("a") == plan.offset("b")
 
 
 def test_smallest_dead_slot_that_fits_and_metrics():
     plan = build(("big", 4096, 0, 0), ("small", 512, 0, 0), ("later", 400, 1, 1),
                  ("wide", 3000, 1, 1))
-    assert plan.at("later").offset == plan.at("small").offset     # not the 4096 one
-    assert plan.at("wide").offset == plan.at("big").offset
-    assert plan.slot_count() == 2
-    assert plan.requested_bytes() == 4096 + 512 + 400 + 3000
-    assert plan.unaliased_bytes() >= plan.requested_bytes()
-    assert plan.reused_bytes() == plan.unaliased_bytes() - plan.total_bytes > 0
+    assert plan.offset("later") == plan.offset("small")     # not the 4096 one
+    assert plan.offset("wide") == plan.offset("big")
+    assert plan.regions() == 2
+    assert plan.bytes_asked() == 4096 + 512 + 400 + 3000
+    assert plan.bytes_without_sharing() >= plan.bytes_asked()
+    assert plan.bytes_saved() == plan.bytes_without_sharing() - plan.arena_bytes > 0
 
 
-def test_requests_and_plans_that_are_refused():
-    planner = WorkspacePlanner()
+def test_requests_and_layouts_that_are_refused():
     for bad in (("", 8, 0, 0), ("x", 0, 0, 0), ("x", 8, 2, 1), ("x", 8, 0, 0, 3), ("x", 8, 0, 0, 0)):
         with pytest.raises(ValueError):
-            planner.add_request(*bad)
-    planner.add_request("x", 8, 0, 0)
-    with pytest.raises(ValueError, match="duplicate"):
-        planner.add_request("x", 8, 1, 1)
-    with pytest.raises(ValueError, match="overlapping live"):
-        WorkspacePlan([Allocation("a", 0, 512, 0, 2), Allocation("b", 256, 512, 1, 3)], 1024)
-    with pytest.raises(ValueError, match="invalid"):
-        WorkspacePlan([Allocation("a", 128, 512, 0, 2)], 1024)          # not aligned
-    with pytest.raises(ValueError, match="invalid"):
-        WorkspacePlan([Allocation("a", 768, 512, 0, 2)], 1024)          # beyond the arena
+            build(bad)
+    with pytest.raises(ValueError, match="twice"):
+        build(("x", 8, 0, 0), ("x", 8, 1, 1))
+    with pytest.raises(ValueError, match="live together"):
+        ArenaLayout([Placement(Lifetime("a", 512, 0, 2), 0),
+                     Placement(Lifetime("b", 512, 1, 3), 256)], 1024)
+    with pytest.raises(ValueError, match="misaligned"):
+        ArenaLayout([Placement(Lifetime("a", 512, 0, 2), 128)], 1024)
+    with pytest.raises(ValueError, match="outside"):
+        ArenaLayout([Placement(Lifetime("a", 512, 0, 2), 768)], 1024)
     with pytest.raises(KeyError):
-        build(("a", 8, 0, 0)).at("b")
+        build(("a", 8, 0, 0)).offset("b")
 
 
 def run_step(ws, signature, sizes=(1000, 600, 1000, 300)):
