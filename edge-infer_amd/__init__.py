@@ -24,16 +24,15 @@ def require_gpu(device="cuda"):
     return torch.device(device)
 
 
-def load_model(model_dir, dtype="bfloat16", device="cuda"):
-    """Build the model that the folder's config.json names, with its weights."""
+def build_model(entry, cfg, tensors, dtype="bfloat16", device="cuda"):
+    """The model of a registered architecture (`entry`, its typed configuration `cfg`) from
+    checkpoint tensors by name: the one assembly behind `load_model` and `api.Model`."""
     from .engine.model import DecoderModel, expected_parameters
-    from .weights import match_parameters, read_tensors
+    from .weights import match_parameters
 
     device = require_gpu(device)
-    entry, cfg, _ = read_config(model_dir)
     spec = cfg.model_spec()
     expected = expected_parameters(spec, cfg.checkpoint_name)
-    tensors = read_tensors(model_dir)
     optional = {"head.weight": "embed.weight"} if spec.tie_word_embeddings else {}
     params = match_parameters(expected, tensors, optional=optional,
                               aliases=getattr(cfg, "checkpoint_aliases", {}))
@@ -41,6 +40,14 @@ def load_model(model_dir, dtype="bfloat16", device="cuda"):
     model = factory(spec, params, dtype, device)
     model.config = cfg
     return model
+
+
+def load_model(model_dir, dtype="bfloat16", device="cuda"):
+    """Build the model that the folder's config.json names, with its weights."""
+    from .weights import read_tensors
+
+    entry, cfg, _ = read_config(model_dir)
+    return build_model(entry, cfg, read_tensors(model_dir), dtype, device)
 
 
 def random_model(cfg, seed, dtype="bfloat16", device="cuda", biases=False):

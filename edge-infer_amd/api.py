@@ -26,49 +26,48 @@ from typing import Mapping, Optional
 
 import torch
 
-from . import require_gpu
+from . import build_model, require_gpu
 from .config import resolve_architecture
 from .engine.generate import generate  # noqa: F401  (re-exported)
-from .engine.model import DecoderModel, expected_parameters
 from .engine.session import Session
 from .sampling.params import SamplingParams  # noqa: F401
-from .weights import match_parameters, read_tensors
+from .weights import read_tensors
 
 MODEL_TYPES = {"qwen3_bf16": "bfloat16", "qwen3_fp32": "float32"}
 DEFAULT_CAPACITY = 4096   # bindings/python/model_bridge.cpp:135-141: min(4096, model limit)
 
 
 def load_checkpoint(model_path, model_type="qwen3_bf16"):
-    """(config dict, {tensor name: tensor}, model type) of a local folder; nothing is
-    ever downloaded (frontend/checkpoint.py:58-105)."""
-    if model_type not in MODEL_TYPES:
-        raise ValueError(f"unsupported model type '{model_type}'; known: {sorted(MODEL_TYPES)}")
-    root = Path(model_path).resolve()
-    with (root / "config.json").open(encoding="utf-8") as source:
-        config = json.load(source)
+    """What `Model` takes, from a local folder: (config.json as a dict, {tensor name:
+    tensor}, model type).  The reference's frontend hands its bridge the same three things
+    (frontend/checkpoint.py:58-105); the tensors here are views of the mapped files."""
+    _known_type(model_type)
+    folder = Path(model_path)
+    config = json.loads((folder / "config.json").read_text(encoding="utf-8"))
     if not isinstance(config, dict):
-        raise ValueError("config.json must hold a JSON object")
-    return config, read_tensors(root), model_type
+        raise ValueError(f"{folder / 'config.json'} must hold a JSON object")
+    return config, read_tensors(folder), model_type
+
+
+def _known_type(model_type) -> str:
+    """The compute type a model type stands for."""
+    try:
+        return MODEL_TYPES[model_type]
+    except (KeyError, TypeError):
+        raise ValueError(f"unsupported model type {model_type!r}; "
+                         f"known: {sorted(MODEL_TYPES)}") from None
 
 
 class Model:
     def __init__(self, config: Mapping, weights: Mapping[str, torch.Tensor],
                  model_type: str = "qwen3_bf16", device: Optional[str] = None):
-        if model_type not in MODEL_TYPES:
-            raise ValueError(f"unsupported model type '{model_type}'; known: {sorted(MODEL_TYPES)}")
+        dtype = _known_type(model_type)
         if device not in (None, "cuda") and not str(device).startswith("cuda"):
             raise ValueError("this library runs on the GPU only (device 'cuda')")
         self._device = require_gpu(device or "cuda")
         entry = resolve_architecture(config)
         self.config = entry.config_class.from_dict(config)
-        spec = self.config.model_spec()
-        expected = expected_parameters(spec, self.config.checkpoint_name)
-        optional = {"head.weight": "embed.weight"} if spec.tie_word_embeddings else {}
-        params = match_parameters(expected, weights, optional=optional,
-                                  aliases=getattr(self.config, "checkpoint_aliases", {}))
-        factory = entry.model_factory or DecoderModel
-        self.decoder = factory(spec, params, MODEL_TYPES[model_type], self._device)
-        self.decoder.config = self.config
+        self.decoder = build_model(entry, self.config, weights, dtype, self._device)
         self.model_type = model_type
 
     @classmethod

@@ -7,7 +7,9 @@ form a group with storage of its own:
 
   key/value group   k, v: [entries, pages, kv_heads, 64, head_dim] in the storage
                     type, a page pool, and per slot the list of its pages
-  state group       [entries, slots, *shape] float32, zeroed when a slot is taken
+  state group       [entries, slots + 1, *shape] float32, zeroed when a slot is taken; the
+                    last row is a spare that no sequence owns (padding of a fixed-size
+                    batch points there, so kernels need no branch for it)
 
 A slot is one live sequence.  Its length is the number of tokens it holds, which is
 also the position of its next token.  Taking a slot leaves old bytes in place: only
@@ -78,9 +80,13 @@ class SessionCache:
             self.kv_k.append(torch.empty(shape, dtype=dtype, device=device))
             self.kv_v.append(torch.empty(shape, dtype=dtype, device=device))
         self.states: List[torch.Tensor] = []
+        self._state_copies: List[torch.Tensor] = []     # [slots, entries, *shape], see save_states
         for request, entries in layout.state_groups:
-            self.states.append(torch.zeros((len(entries), self.n_slots) + tuple(request.shape),
+            self.states.append(torch.zeros((len(entries), self.n_slots + 1) + tuple(request.shape),
                                            dtype=torch.float32, device=device))
+            self._state_copies.append(torch.empty((self.n_slots, len(entries))
+                                                  + tuple(request.shape),
+                                                  dtype=torch.float32, device=device))
 
     # -- slots -------------------------------------------------------------
     def acquire(self) -> int:
@@ -130,6 +136,20 @@ class SessionCache:
             for pages in self.kv_pages:
                 pages.trim(slot, new_length)
 
+    # -- fixed-size state: what a step may change in place ------------------
+    def save_states(self, slots: torch.Tensor) -> None:
+        """Copy the state rows of these slots (int32 on the device, one per live sequence of
+        the step about to run) aside.  Mixers update state in place while a step runs; keys
+        and values of a failed step lie beyond the committed lengths and are simply written
+        again, but state has no such place, so a failed step puts these copies back."""
+        for state, copy in zip(self.states, self._state_copies):
+            torch.index_select(state.transpose(0, 1), 0, slots, out=copy[:slots.numel()])
+
+    def restore_states(self, slots: torch.Tensor) -> None:
+        """Put back what `save_states` copied for the same slots."""
+        for state, copy in zip(self.states, self._state_copies):
+            state.transpose(0, 1).index_copy_(0, slots.long(), copy[:slots.numel()])
+
     # -- views -------------------------------------------------------------
     def kv(self, cache_id: int):
         kind, group, index = self.layout.entry_group[cache_id]
@@ -138,7 +158,8 @@ class SessionCache:
         return group, self.kv_k[group][index], self.kv_v[group][index]
 
     def state(self, cache_id: int) -> torch.Tensor:
-        """[slots, *shape] float32 of a fixed-size state entry."""
+        """[slots + 1, *shape] float32 of a fixed-size state entry (row = slot; the last row
+        is the spare one)."""
         kind, group, index = self.layout.entry_group[cache_id]
         if kind != "state":
             raise KeyError(f"cache entry {cache_id} holds no fixed-size state")
@@ -156,7 +177,7 @@ class SessionCache:
 
     def bytes(self) -> int:
         total = 0
-        for tensor in self.kv_k + self.kv_v + self.states:
+        for tensor in self.kv_k + self.kv_v + self.states + self._state_copies:
             total += tensor.numel() * tensor.element_size()
         return total
 

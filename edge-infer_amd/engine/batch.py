@@ -1,21 +1,30 @@
 """Row metadata of one step: built on the host, uploaded in one copy.
 
-A step runs the tokens it is given as one packed batch of rows.  Only position
-encoding, cache store and attention read the metadata; every other operation is
-row-wise.  All of it lives in one int32 buffer:
+A step runs the tokens it is given as one packed batch of rows.  Row-wise operations
+never read the metadata; position encoding, cache stores and mixers do.  All of it lives
+in one int32 buffer of named sections:
 
-  longest[1] tokens[N] row_pos[N] row_seq[N] want_rows[W]
-  per attention item size: item_seq[I] item_row0[I] item_npos[I]   (prefill)
-  decode items: item_seq[B] item_row0[B] item_npos[B]             (decode)
-  per key/value group: page_table[B, width]
+  longest[1]                           most tokens any sequence holds after the step
+  tokens[N] row_pos[N] row_seq[N]      per row: token id, position, index of its sequence
+  want_rows[W]                         rows whose logits are wanted
+  seq_slot[B] seq_start[B] seq_count[B]  per sequence: cache slot (its row in every state
+                                       table), tokens held before the step, tokens brought
+  pages<g>[B, width]                   per key/value group: logical page -> physical page
+  ...                                  whatever the model's parts plan for themselves
 
-Padding rows (a fixed-size decode batch with fewer live sequences) carry
-row_seq = -1, want_rows = -1 and items with seq = -1: kernels skip them.
+The last kind is the parts' own: a part with a `plan_step(plan)` method returns
+`{section name: int32 array}` (work items of its kernels, for instance) and finds them
+again on the device as `ctx.meta.section(name)`.  The engine does not know what they mean.
+
+Padding (a decode batch of fixed size with fewer live sequences) carries row_seq = -1,
+want_rows = -1 and seq_count = 0: kernels skip such rows and sequences.  Its seq_slot is the
+spare slot, a row that every state table has beyond the rows of the real slots and that no
+sequence ever owns: a kernel may read and write it without a branch.
 """
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import Dict, List, Mapping, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -35,10 +44,14 @@ class SeqStep:
 
 
 class StepPlan:
-    """Host-side description of a step, independent of any device."""
+    """Host-side description of a step, independent of any device.
 
-    def __init__(self, seqs: List[SeqStep], item_sizes: Sequence[int] = (),
-                 pad_seqs: Optional[int] = None):
+    `context_bound`: the launch shapes of this step must hold for sequences of up to that
+    many tokens (a captured step is replayed for every context up to its bound); by default
+    the longest sequence of the step itself."""
+
+    def __init__(self, seqs: List[SeqStep], pad_seqs: Optional[int] = None,
+                 context_bound: Optional[int] = None, spare_slot: int = -1):
         if not seqs:
             raise ValueError("a step needs at least one sequence")
         self.seqs = seqs
@@ -60,17 +73,26 @@ class StepPlan:
         self.n_rows = self.n_seqs if pad_seqs is not None else row
         self.padded = pad_seqs is not None
         self.max_context = max(seq.start + seq.count for seq in seqs)
+        self.context_bound = self.max_context if context_bound is None else int(context_bound)
+        if self.context_bound < self.max_context:
+            raise ValueError("the context bound of a step is below its longest sequence")
 
         n = self.n_rows
         self.tokens = np.zeros(n, dtype=np.int32)
         self.row_pos = np.zeros(n, dtype=np.int32)
         self.row_seq = np.full(n, -1, dtype=np.int32)
+        self.seq_slot = np.full(self.n_seqs, spare_slot, dtype=np.int32)
+        self.seq_start = np.zeros(self.n_seqs, dtype=np.int32)
+        self.seq_count = np.zeros(self.n_seqs, dtype=np.int32)
         want_rows: List[int] = []
         for index, seq in enumerate(seqs):
             rows = slice(seq.row0, seq.row0 + seq.count)
             self.tokens[rows] = np.asarray(seq.tokens, dtype=np.int64)
             self.row_pos[rows] = np.arange(seq.start, seq.start + seq.count)
             self.row_seq[rows] = index
+            self.seq_slot[index] = seq.slot
+            self.seq_start[index] = seq.start
+            self.seq_count[index] = seq.count
             for w in seq.want:
                 if not 0 <= w < seq.count:
                     raise ValueError(f"wanted place {w} is outside the {seq.count} tokens given")
@@ -80,47 +102,30 @@ class StepPlan:
             # a fixed-size decode batch asks for every row; dead rows are marked -1
             want_rows = [seq.row0 for seq in seqs] + [-1] * (self.n_seqs - len(seqs))
         self.want_rows = np.asarray(want_rows, dtype=np.int32)
-        self.item_sizes = tuple(sorted(set(item_sizes)))
-        self.items: Dict[int, Tuple[np.ndarray, np.ndarray, np.ndarray]] = {}
-        if not self.decode:
-            for size in self.item_sizes:
-                self.items[size] = self._prefill_items(size)
+        self.extra: Dict[str, np.ndarray] = {}
 
-    def _prefill_items(self, size: int):
-        """(sequence, first row, positions) of every work item, the ones with the longest
-        key range first: they take longest, so they should start first."""
-        items = []
-        for index, seq in enumerate(self.seqs):
-            for p0 in range(0, seq.count, size):
-                npos = min(size, seq.count - p0)
-                items.append((-(seq.start + p0 + npos), index, seq.row0 + p0, npos))
-        items.sort()
-        return (np.asarray([i[1] for i in items], dtype=np.int32),
-                np.asarray([i[2] for i in items], dtype=np.int32),
-                np.asarray([i[3] for i in items], dtype=np.int32))
-
-    def decode_items(self):
-        seq = np.full(self.n_seqs, -1, dtype=np.int32)
-        seq[:self.n_live_seqs] = np.arange(self.n_live_seqs)
-        row0 = np.arange(self.n_seqs, dtype=np.int32)
-        npos = np.zeros(self.n_seqs, dtype=np.int32)
-        npos[:self.n_live_seqs] = 1
-        return seq, row0, npos
+    def add_sections(self, sections: Mapping[str, np.ndarray]) -> None:
+        """Sections that a part planned for itself.  Parts of one kind may plan the same
+        section; it is kept once."""
+        for name, array in sections.items():
+            array = np.ascontiguousarray(array, dtype=np.int32)
+            held = self.extra.get(name)
+            if held is not None and not np.array_equal(held, array):
+                raise ValueError(f"two parts planned different contents for the section '{name}'")
+            self.extra[name] = array
 
     def sections(self, page_tables: Sequence[np.ndarray]) -> List[Tuple[str, np.ndarray]]:
-        # longest: the most tokens any sequence holds after this step (decode attention sizes
-        # its slices by it); first, so that its place never depends on the batch
+        # `longest` comes first, so that its place never depends on the batch
         out = [("longest", np.asarray([self.max_context], dtype=np.int32)),
                ("tokens", self.tokens), ("row_pos", self.row_pos), ("row_seq", self.row_seq),
-               ("want_rows", self.want_rows)]
-        if self.decode:
-            seq, row0, npos = self.decode_items()
-            out += [("ditem_seq", seq), ("ditem_row0", row0), ("ditem_npos", npos)]
-        for size, (seq, row0, npos) in self.items.items():
-            out += [(f"item{size}_seq", seq), (f"item{size}_row0", row0),
-                    (f"item{size}_npos", npos)]
+               ("want_rows", self.want_rows), ("seq_slot", self.seq_slot),
+               ("seq_start", self.seq_start), ("seq_count", self.seq_count)]
         for index, table in enumerate(page_tables):
             out.append((f"pages{index}", table.reshape(-1)))
+        for name, array in self.extra.items():
+            if any(name == taken for taken, _ in out):
+                raise ValueError(f"a part planned a section under the engine's name '{name}'")
+            out.append((name, array.reshape(-1)))
         return out
 
 
@@ -143,6 +148,11 @@ class DeviceMeta:
             self._device_buffer = torch.empty(size, dtype=torch.int32, device=self.device)
             pin = self.device is not None and torch.device(self.device).type == "cuda"
             self._host_buffer = torch.empty(size, dtype=torch.int32, pin_memory=pin)
+
+    @property
+    def capacity(self) -> int:
+        """int32 elements the device buffer holds (0 before the first upload)."""
+        return 0 if self._device_buffer is None else self._device_buffer.numel()
 
     def upload(self, plan: StepPlan, page_tables: Sequence[np.ndarray]) -> None:
         sections = plan.sections(page_tables)
@@ -167,33 +177,29 @@ class DeviceMeta:
         self.n_want = int(plan.want_rows.size)
 
     # views ------------------------------------------------------------
-    @property
-    def longest(self):
-        return self._views["longest"]
+    def section(self, name: str) -> torch.Tensor:
+        """int32 view of a named section on the device."""
+        try:
+            return self._views[name]
+        except KeyError:
+            raise KeyError(f"the step's metadata holds no section '{name}'; "
+                           f"it holds {sorted(self._views)}") from None
 
-    @property
-    def tokens(self):
-        return self._views["tokens"]
+    def layout(self):
+        """(name, offset, size) of every section: two uploads with the same layout leave
+        every view where it was (what a captured step relies on)."""
+        base = self._device_buffer.data_ptr()
+        return tuple((name, (view.data_ptr() - base) // 4, view.numel())
+                     for name, view in self._views.items())
 
-    @property
-    def row_pos(self):
-        return self._views["row_pos"]
-
-    @property
-    def row_seq(self):
-        return self._views["row_seq"]
-
-    @property
-    def want_rows(self):
-        return self._views["want_rows"]
+    longest = property(lambda self: self.section("longest"))
+    tokens = property(lambda self: self.section("tokens"))
+    row_pos = property(lambda self: self.section("row_pos"))
+    row_seq = property(lambda self: self.section("row_seq"))
+    want_rows = property(lambda self: self.section("want_rows"))
+    seq_slot = property(lambda self: self.section("seq_slot"))
+    seq_start = property(lambda self: self.section("seq_start"))
+    seq_count = property(lambda self: self.section("seq_count"))
 
     def page_table(self, group: int) -> torch.Tensor:
-        return self._views[f"pages{group}"].view(self.n_seqs, self._table_widths[group])
-
-    def decode_items(self):
-        return (self._views["ditem_seq"], self._views["ditem_row0"], self._views["ditem_npos"],
-                self.n_seqs)
-
-    def prefill_items(self, size: int):
-        seq = self._views[f"item{size}_seq"]
-        return seq, self._views[f"item{size}_row0"], self._views[f"item{size}_npos"], seq.numel()
+        return self.section(f"pages{group}").view(self.n_seqs, self._table_widths[group])

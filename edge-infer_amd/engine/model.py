@@ -54,6 +54,56 @@ def expected_parameters(spec: ModelSpec, checkpoint_name: Callable[[str], str]
             for path, param in model_parameters(spec).items()}
 
 
+def _round_up_fine(count: int) -> int:
+    """The next multiple of an eighth of the power of two at or below `count`: at most an
+    eighth above it."""
+    if count <= 8:
+        return count
+    step = 1 << (count.bit_length() - 4)
+    return (count + step - 1) // step * step
+
+
+def _round_up_coarse(count: int) -> int:
+    return 1 << max(0, (count - 1).bit_length())
+
+
+FEW_ROWS = 256
+
+
+def workspace_class(ctx):
+    """(signature, scale) under which a step's buffers are planned.  Decode steps and steps
+    of few rows are planned for their exact shape (the few-rows product slices K differently
+    for every row count).  Prompt steps of more rows share a plan with every step of about
+    their size: rows rounded up by at most an eighth, sequences and wanted rows to a power of
+    two (wanted rows that are all rows follow the rows); the recorded sizes are scaled to the
+    largest step of the class, which is safe because every buffer of such a step is at most
+    linear in rows, sequences and wanted rows."""
+    rows, seqs, want = ctx.n_rows, ctx.n_seqs, ctx.meta.n_want
+    bound = ctx.context_bound if ctx.fixed_shape else None
+    if ctx.decode or rows <= FEW_ROWS:
+        return (rows, seqs, want, ctx.decode, bound), 1.0
+    rows_up, seqs_up = _round_up_fine(rows), _round_up_coarse(seqs)
+    if want == rows:
+        want_up, want_key = rows_up, "all"
+    elif want == 0:
+        want_up = want_key = 0
+    else:
+        want_up = want_key = _round_up_coarse(want)
+    scale = max(rows_up / rows, seqs_up / seqs, want_up / max(1, want))
+    return (rows_up, seqs_up, want_key, False, bound), scale
+
+
+def members_of(block):
+    """The parts a block holds: what its `members()` names, or else every attribute of it
+    that is a part (has `forward` or `add_norm`).  The model asks them, not the block, what
+    they plan for a step and whether they can be captured, so a block arrangement is only
+    an order of calls."""
+    if hasattr(block, "members"):
+        return tuple(block.members())
+    return tuple(part for part in vars(block).values()
+                 if hasattr(part, "forward") or hasattr(part, "add_norm"))
+
+
 class DecoderModel:
     def __init__(self, spec: ModelSpec, params: Mapping[str, torch.Tensor], dtype, device):
         spec.validate()
@@ -93,14 +143,6 @@ class DecoderModel:
             self._positions[position_spec] = table
         return table
 
-    def attention_item_sizes(self):
-        sizes = set()
-        for layer in self.layers:
-            mixer = getattr(layer, "mixer", None)
-            if mixer is not None and hasattr(mixer, "positions_per_item"):
-                sizes.add(mixer.positions_per_item())
-        return tuple(sorted(sizes))
-
     def max_positions(self) -> int:
         limit = self.spec.max_position_embeddings
         for table in self._positions.values():
@@ -108,34 +150,31 @@ class DecoderModel:
                 limit = min(limit, table.max_positions)
         return limit
 
-    def capture_safe(self) -> bool:
-        """Whether a decode step may be captured in a HIP graph: every block and every
-        part that a block holds (norms, mixer, feed-forward) must say so with
-        `capture_safe = True` (it launches nothing but capturable kernels and allocates
-        nothing per step; a part that does not say so is taken to be unsafe), and every
-        linear layer must take the hand-written kernel for few rows (library products may
-        record memset nodes, which are not replayed reliably)."""
-        def linears(obj, depth=0):
-            if isinstance(obj, Linear):
-                yield obj
-            elif depth < 3 and hasattr(obj, "__dict__"):
-                for value in vars(obj).values():
-                    yield from linears(value, depth + 1)
-        if not getattr(self.final_norm, "capture_safe", False):
-            return False
+    def plan_step(self, plan) -> None:
+        """Let every part add the metadata sections it plans for itself (work items of its
+        kernels and the like) to the step plan; the engine only carries them."""
         for layer in self.layers:
-            if not getattr(layer, "capture_safe", False):
-                return False
-            for part in vars(layer).values():
-                if hasattr(part, "forward") or hasattr(part, "add_norm"):
-                    if not getattr(part, "capture_safe", False):
-                        return False
-            for linear in linears(layer):
-                if linear.dtype == torch.bfloat16 and linear.in_features % 8:
-                    return False
-        if self.head.dtype == torch.bfloat16 and self.head.in_features % 8:
-            return False
-        return True
+            for part in (layer, *members_of(layer)):
+                if hasattr(part, "plan_step"):
+                    plan.add_sections(part.plan_step(plan))
+
+    def capture_safe(self) -> bool:
+        """Whether a decode step may be captured in a HIP graph: the final norm, the head,
+        every block and every part of a block must say so with `capture_safe` (it launches
+        nothing but capturable kernels and allocates nothing per step; a part that does not
+        say so is taken to be unsafe)."""
+        parts = [self.final_norm, self.head]
+        for layer in self.layers:
+            parts += [layer, *members_of(layer)]
+        return all(bool(getattr(part, "capture_safe", False)) for part in parts)
+
+    def capture_rows(self) -> int:
+        """Most rows of a step for which `capture_safe` holds: the least any part allows."""
+        rows = self.head.capture_rows
+        for layer in self.layers:
+            for part in (layer, *members_of(layer)):
+                rows = min(rows, getattr(part, "capture_rows", 1 << 30))
+        return rows
 
     def weight_bytes(self) -> int:
         seen, total = set(), 0
@@ -162,8 +201,7 @@ class DecoderModel:
         are planned by the workspace per shape of step: rows, sequences, wanted rows, kind,
         and the context bound that fixes the launch shape of decode attention."""
         workspace = ctx.workspace
-        workspace.start((ctx.n_rows, ctx.n_seqs, ctx.meta.n_want, ctx.decode,
-                         getattr(ctx, "_fixed_context", None)))
+        workspace.start(*workspace_class(ctx))
         try:
             logits = self._forward(ctx)
         except BaseException:

@@ -11,58 +11,40 @@ from __future__ import annotations
 
 import numbers
 import os
-from typing import Dict, List, Optional, Sequence, Tuple
+from collections import OrderedDict
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
 from ..cache.allocator import PAGE_TOKENS
 from ..cache.storage import CacheLayout, SessionCache
 from ..parts.base import StepContext, Workspace
-from ..parts.linear import SKINNY_ROWS
 from .batch import DeviceMeta, SeqStep, StepPlan
 
+# EDGE_INFER_DECODE_GRAPHS=0: decode steps run eagerly instead of from HIP graphs (the
+# reference has such a switch too, runtime/src/qwen3.cpp:9-12, where graphs are off unless set)
+GRAPHS_SWITCH = "EDGE_INFER_DECODE_GRAPHS"
+MAX_GRAPHS = 24         # captured decode steps a session keeps; the one unused for longest goes
 
-class _Context(StepContext):
-    def __init__(self, session, fixed_context=None, **kwargs):
-        super().__init__(**kwargs)
-        self._session = session
-        self._fixed_context = fixed_context
 
-    def decode_splits(self, n_kv_heads: int) -> int:
-        """How many blocks share the key range of one (sequence, kv head) in decode:
-        enough to put about two blocks on each of the 256 compute units, never more
-        than there are pages.  A captured step fixes the count by the capacity (blocks
-        whose share of a short sequence is empty return at once)."""
-        context = self._fixed_context or self.max_context
-        pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
-        blocks = self.n_seqs * n_kv_heads
-        wanted = (512 + blocks - 1) // blocks
-        return max(1, min(wanted, pages, 32))
+def batch_bucket(live: int) -> int:
+    """The fixed batch size a decode step of `live` sequences is padded to when it is
+    captured: powers of two up to 64, then multiples of 32."""
+    bucket = 1
+    while bucket < live and bucket < 64:
+        bucket *= 2
+    return bucket if bucket >= live else (live + 31) // 32 * 32
 
-    def decode_plan(self, n_kv_heads: int, group: int = 1):
-        """(slices, waves per block) for the matrix-core decode kernel.  Up to 256 (sequence,
-        kv head) pairs: blocks of 16 waves, a tile of 16 keys per wave at a time, and as many
-        slices of the key range as shorten a wave's walk by more than the merge kernel costs,
-        while all blocks still fit the chip at once (256 compute units x 16 waves).  The
-        weights are measured ones: 1.9 us for a tile a wave walks, 4.5 us for the merge and
-        0.1 us for each slice it reads.  More pairs than that: blocks of 4 waves, see
-        `decode_splits`."""
-        context = self._fixed_context or self.max_context
-        # (a block of 16 waves takes at most 4 query heads of a group: larger groups have
-        # several blocks per pair)
-        pairs = self.n_seqs * n_kv_heads * ((group + 3) // 4)
-        if pairs > 256:
-            return self.decode_splits(n_kv_heads), 4
-        tiles = (context + 15) // 16
-        pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
-        best, best_cost = 1, 1.9 * ((tiles + 15) // 16)
-        slices = 2
-        while slices <= min(pages, 32) and pairs * 16 * slices <= 4096:
-            cost = 1.9 * ((tiles + 16 * slices - 1) // (16 * slices)) + 4.5 + 0.1 * slices
-            if cost < best_cost:
-                best, best_cost = slices, cost
-            slices *= 2
-        return best, 16
+
+def context_bound(context: int, capacity: int) -> int:
+    """The bound a captured decode step holds for: the next of 256, 384, 512, 768, 1024,
+    1536, ... at or above the longest sequence, capped by the capacity.  Parts fix their
+    launch shapes by the bound (see `StepContext.context_bound`), so finer steps mean shapes
+    that fit the true lengths better, at the price of more graphs."""
+    bound = 256
+    while bound < context:
+        bound = bound * 3 // 2 if bound & (bound - 1) == 0 else bound // 3 * 4
+    return max(1, min(bound, capacity))
 
 
 class _CapturedDecode:
@@ -75,6 +57,9 @@ class _CapturedDecode:
         self.workspace = Workspace(device)
         self.graph = None
         self.logits = None
+        self.layout = None      # where the metadata sections lay when the graph was captured
+        self.plan = None        # the step about to run
+        self.key = None         # (batch bucket, context bound)
 
 
 class Session:
@@ -100,16 +85,17 @@ class Session:
         self._sampler = None
         self.workspace = Workspace(self.device)
         self.meta = DeviceMeta(self.device)
-        self._item_sizes = model.attention_item_sizes()
         self.steps_run = 0
         # decode steps are replayed from HIP graphs unless the model has an operation
         # that is not safe to capture (see DecoderModel.capture_safe) or the caller or the
-        # environment says no: EDGE_INFER_ENABLE_QWEN3_GRAPH=0 (the reference's switch,
-        # runtime/src/qwen3.cpp:9-12, where graphs are off unless it is 1)
-        self.graphs = (bool(graphs) and os.environ.get("EDGE_INFER_ENABLE_QWEN3_GRAPH", "1") != "0"
+        # environment says no
+        self.graphs = (bool(graphs) and os.environ.get(GRAPHS_SWITCH, "1") != "0"
                        and model.capture_safe())
-        self._captured: Dict[Tuple[int, int], _CapturedDecode] = {}
+        self._capture_rows = min(model.capture_rows(), 256) if self.graphs else 0
+        self._captured: "OrderedDict[Tuple[int, int], _CapturedDecode]" = OrderedDict()
+        self._graph_logits = None     # one buffer for the logits of every captured step
         self.graph_replays = 0
+        self.graph_captures = 0
         # one generation or reset at a time: a callback that calls back into its own session
         # is refused, as in the reference (bindings/python/include/python_callback.hpp:16-26)
         self._busy = False
@@ -125,13 +111,19 @@ class Session:
         """Give a slot and everything it holds back."""
         self.cache.release(slot)
 
-    def reset(self) -> None:
-        """End every live sequence; allocations are kept."""
+    def reset(self, trim: bool = False) -> None:
+        """End every live sequence.  Allocations are kept unless `trim` is set: then the step
+        workspaces and the captured graphs go too (the cache stays), which gives back what a
+        single very large step made the session hold."""
         if self._busy:
             raise RuntimeError("the session is busy; wait for the current operation to finish")
         self._require_usable()
         torch.cuda.synchronize(self.device)
         self.cache.release_all()
+        if trim:
+            self._captured.clear()
+            self._graph_logits = None
+            self.workspace.clear()
 
     def length(self, slot: int) -> int:
         if not self.cache.slots.is_live(slot):
@@ -159,11 +151,11 @@ class Session:
         values would need without sharing, and what sharing saves (the reference reports
         the same of its decode plan, runtime/include/qwen3.hpp:60-63)."""
         def plans(workspace):
-            return {signature: {"arena_bytes": layout.plan.total_bytes,
-                                "unaliased_bytes": layout.plan.unaliased_bytes(),
-                                "reused_bytes": layout.plan.reused_bytes(),
-                                "values": len(layout.plan.allocations),
-                                "slots": layout.plan.slot_count()}
+            return {signature: {"arena_bytes": layout.arena.arena_bytes,
+                                "bytes_without_sharing": layout.arena.bytes_without_sharing(),
+                                "bytes_saved": layout.arena.bytes_saved(),
+                                "buffers": len(layout.arena),
+                                "regions": layout.arena.regions()}
                     for signature, layout in workspace._plans.items()}
         report = {"held_bytes": self.workspace.bytes(), "plans": plans(self.workspace)}
         for key, captured in self._captured.items():
@@ -259,17 +251,26 @@ class Session:
         growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
         self.cache.check_growth(growth)          # raises before anything changes
         self.cache.grow(growth)
+        saved = None
         try:
-            # batches beyond the few-rows product's reach multiply through the library, whose
-            # kernels are kept out of graphs
-            if (self.graphs and len(seqs) <= SKINNY_ROWS
+            captured = None
+            if (self.graphs and batch_bucket(len(seqs)) <= self._capture_rows
                     and all(seq.count == 1 for seq in seqs)):
-                logits = self._run_captured(seqs)
+                captured = self._captured_for(seqs)
+            if captured is None:
+                plan = self._plan(seqs)
+                meta, workspace = self.meta, self.workspace
             else:
-                plan = StepPlan(seqs, item_sizes=self._item_sizes)
-                logits = self._run(plan, self.meta, self.workspace)
+                plan, meta, workspace = captured.plan, captured.meta, captured.workspace
+            ctx = self._context(plan, meta, workspace, fixed_shape=captured is not None)
+            if self.cache.states:
+                # state of fixed size is updated in place: keep what the step may change
+                saved = meta.seq_slot[:plan.n_live_seqs]
+                self.cache.save_states(saved)
+            logits = (self.model.forward(ctx) if captured is None
+                      else self._run_captured(captured, ctx))
         except BaseException:
-            self._drain_failed_step()
+            self._drain_failed_step(saved)
             raise                                 # the original error
         self.cache.commit(growth)
         self.steps_run += 1
@@ -279,52 +280,79 @@ class Session:
         if self._unusable:
             raise RuntimeError("the session is unusable after a failed GPU stream completion")
 
-    def _drain_failed_step(self) -> None:
+    def _drain_failed_step(self, saved_slots=None) -> None:
         """After an error in a step that may have launched work: wait for what was launched.
-        The sequences keep the lengths they had (what the step wrote lies beyond them and
-        is written again by the next step), so the session stays usable; only if the wait
-        itself fails is nothing known any more, and the session refuses every later call,
-        as the reference's does (runtime/src/qwen3.cpp:126-161,374-379)."""
+        The sequences keep the lengths they had: keys and values that the step wrote lie
+        beyond them and are written again by the next step, and state of fixed size, which
+        mixers update in place, is put back from the copy taken before the step.  So the
+        session stays usable; only if the wait or the restoring itself fails is nothing known
+        any more, and the session refuses every later call, as the reference's does
+        (runtime/src/qwen3.cpp:126-161,374-379)."""
         try:
             torch.cuda.synchronize(self.device)
+            if saved_slots is not None:
+                self.cache.restore_states(saved_slots)
+                torch.cuda.synchronize(self.device)
         except Exception:       # the original error is the one that is raised
             self._unusable = True
 
-    def _context(self, plan, meta, workspace, fixed_context=None):
+    def _plan(self, seqs, pad_seqs=None, bound=None) -> StepPlan:
+        plan = StepPlan(seqs, pad_seqs=pad_seqs, context_bound=bound,
+                        spare_slot=self.cache.n_slots)
+        self.model.plan_step(plan)      # the parts add the sections they plan for themselves
+        return plan
+
+    def _context(self, plan, meta, workspace, fixed_shape=False):
         slots = [seq.slot for seq in plan.seqs]
         tables = [self.cache.page_rows(group, slots, plan.n_seqs)
                   for group in range(len(self.cache.kv_pages))]
         meta.upload(plan, tables)
-        ctx = _Context(self, fixed_context=fixed_context, dtype=self.dtype, device=self.device,
-                       n_rows=plan.n_rows, n_seqs=plan.n_seqs, decode=plan.decode, meta=meta,
-                       cache=self.cache, workspace=workspace, max_context=plan.max_context)
+        ctx = StepContext(dtype=self.dtype, device=self.device, n_rows=plan.n_rows,
+                          n_seqs=plan.n_seqs, decode=plan.decode, meta=meta, cache=self.cache,
+                          workspace=workspace, max_context=plan.max_context,
+                          context_bound=plan.context_bound, fixed_shape=fixed_shape)
         ctx.sequences = plan.seqs
         return ctx
 
-    def _run(self, plan: StepPlan, meta: DeviceMeta, workspace: Workspace) -> torch.Tensor:
-        return self.model.forward(self._context(plan, meta, workspace))
+    def context_for(self, seqs: List[SeqStep]):
+        """(step context, plan) for these sequences on the session's own buffers, with the
+        metadata uploaded and nothing run: what a part needs to be driven on its own."""
+        plan = self._plan(seqs)
+        return self._context(plan, self.meta, self.workspace), plan
 
-    def _run_captured(self, seqs: List[SeqStep]) -> torch.Tensor:
-        """A decode step through the graph of its batch-size bucket (powers of two up to
-        64, then steps of 32) and context bound.  The first step of a bucket runs eagerly on the bucket's own buffers
-        and is then captured; later steps only refresh the metadata and replay."""
-        live = len(seqs)
-        bucket = 1
-        while bucket < live and bucket < 64:
-            bucket *= 2
-        if bucket < live:
-            bucket = (live + 31) // 32 * 32
-        plan = StepPlan(seqs, item_sizes=self._item_sizes, pad_seqs=bucket)
-        # the launch shapes of attention depend on how long the sequences may be: a graph
-        # holds for contexts up to a bound (1,024, 4,096, ... or the capacity)
-        bound = 1024
-        while bound < plan.max_context:
-            bound *= 4
-        bound = min(bound, self.capacity)
-        captured = self._captured.get((bucket, bound))
+    def _captured_for(self, seqs: List[SeqStep]) -> _CapturedDecode:
+        """The captured step for this batch: one per batch-size bucket and context bound,
+        the most recently used `MAX_GRAPHS` of them.  All of them write their logits into one
+        buffer of the session (the next step overwrites a step's logits anyway)."""
+        bucket = batch_bucket(len(seqs))
+        longest = max(seq.start + seq.count for seq in seqs)
+        bound = context_bound(longest, self.capacity)
+        key = (bucket, bound)
+        captured = self._captured.pop(key, None)
         if captured is None:
-            captured = self._captured[(bucket, bound)] = _CapturedDecode(self.device)
-        ctx = self._context(plan, captured.meta, captured.workspace, fixed_context=bound)
+            captured = _CapturedDecode(self.device)
+            while len(self._captured) >= MAX_GRAPHS:
+                self._captured.popitem(last=False)
+        self._captured[key] = captured
+        vocab = self.model.spec.vocab_size
+        rows = batch_bucket(min(self.max_batch, self._capture_rows))
+        if self._graph_logits is None or self._graph_logits.numel() < bucket * vocab:
+            self._captured.clear()          # graphs hold the old buffer's address
+            self._captured[key] = captured = _CapturedDecode(self.device)
+            self._graph_logits = torch.empty(max(rows, bucket) * vocab, dtype=torch.float32,
+                                             device=self.device)
+        captured.workspace.bind("logits", self._graph_logits)
+        captured.plan = self._plan(seqs, pad_seqs=bucket, bound=bound)
+        captured.key = key
+        return captured
+
+    def _run_captured(self, captured: _CapturedDecode, ctx) -> torch.Tensor:
+        """The first step of a (bucket, bound) pair runs eagerly on the pair's own buffers and
+        is then captured; later steps only refresh the metadata and replay."""
+        seqs = ctx.sequences
+        layout = (captured.meta.layout(), captured.meta.capacity)
+        if captured.graph is not None and captured.layout != layout:
+            captured.graph = None           # the metadata moved: what was captured reads stale places
         if captured.graph is None:
             try:
                 logits = self.model.forward(ctx)
@@ -333,17 +361,18 @@ class Session:
                 with torch.cuda.graph(graph):
                     captured.logits = self.model.forward(ctx)
             except BaseException:
-                self._captured.pop((bucket, bound), None)   # nothing half-made is kept
+                self._captured.pop(captured.key, None)   # nothing half-made is kept
                 raise
-            captured.graph = graph
+            captured.graph, captured.layout = graph, layout
+            self.graph_captures += 1
         else:
             captured.graph.replay()
             self.graph_replays += 1
             logits = captured.logits
         # the captured step computes the logits of every row; hand out the wanted ones
-        wanted = [index for index, seq in enumerate(seqs) if len(seq.want) > 0]
-        if len(wanted) == live:
-            return logits[:live]
-        if not wanted:
+        rows = [index for index, seq in enumerate(seqs) for _ in seq.want]
+        if rows == list(range(len(seqs))):
+            return logits[:len(seqs)]
+        if not rows:
             return logits[:0]
-        return logits[torch.tensor(wanted, device=self.device)]
+        return logits[torch.tensor(rows, device=self.device)]

@@ -12,9 +12,11 @@ from __future__ import annotations
 
 import os
 
+import numpy as np
 import torch
 
 from ..csrc import lib
+from ..csrc.lib import PAGE_TOKENS
 from ..weights.loader import ParamSpec
 from .base import KVRequest
 from .linear import Linear
@@ -24,8 +26,23 @@ from .linear import Linear
 FUSED_DECODE = os.environ.get("EDGE_INFER_FUSED_DECODE", "1") != "0"
 
 
+# What the matrix-core decode kernel costs, measured on an MI355X (head size 128): a wave
+# walks a tile of 16 keys in 1.9 us; merging slices costs 4.5 us and 0.1 us a slice.
+TILE_US, MERGE_US, MERGE_SLICE_US = 1.9, 4.5, 0.1
+WAVE_SLOTS = 256 * 16         # waves the chip holds at once: compute units x waves a unit
+MAX_SLICES = 32
+
+
 class Attention:
-    capture_safe = True   # launches only this library's kernels; nothing allocates per step
+    @property
+    def capture_safe(self):
+        """Launches only this library's kernels and allocates nothing per step, as long as
+        its products do."""
+        return self.qkv.capture_safe and self.o.capture_safe
+
+    @property
+    def capture_rows(self):
+        return min(self.qkv.capture_rows, self.o.capture_rows)
 
     @classmethod
     def parameters(cls, spec, hidden):
@@ -92,6 +109,67 @@ class Attention:
             return lib.attention_prefill_mfma_positions(self.group)
         return lib.attention_positions_per_item(self.group)
 
+    def _items_section(self):
+        return f"attention.items{self.positions_per_item()}"
+
+    def plan_step(self, plan):
+        """The work items of this step's attention kernels, as one int32 section [3, items]:
+        sequence (-1: padding), first row, positions.  A prompt step cuts every sequence's
+        rows into items of `positions_per_item`, the ones with the longest key range first
+        (they take longest, so they start first); a decode step has one item a sequence."""
+        if plan.decode:
+            seq = np.full(plan.n_seqs, -1, dtype=np.int32)
+            seq[:plan.n_live_seqs] = np.arange(plan.n_live_seqs)
+            npos = np.zeros(plan.n_seqs, dtype=np.int32)
+            npos[:plan.n_live_seqs] = 1
+            items = np.stack([seq, np.arange(plan.n_seqs, dtype=np.int32), npos])
+            return {"attention.decode_items": items}
+        size = self.positions_per_item()
+        items = []
+        for index, seq in enumerate(plan.seqs):
+            for p0 in range(0, seq.count, size):
+                npos = min(size, seq.count - p0)
+                items.append((-(seq.start + p0 + npos), index, seq.row0 + p0, npos))
+        items.sort()
+        return {self._items_section(): np.asarray([item[1:] for item in items],
+                                                  dtype=np.int32).T.copy()}
+
+    @staticmethod
+    def _items(ctx, name):
+        section = ctx.meta.section(name)
+        count = section.numel() // 3
+        return section[:count], section[count:2 * count], section[2 * count:], count
+
+    def decode_launch(self, n_seqs: int, context: int):
+        """(slices of the key range, waves a block) of a decode step over `n_seqs` sequences
+        of up to `context` tokens.  A slice is the same number of pages for every sequence.
+
+        Matrix-core kernel, up to 256 (sequence, kv head) pairs: blocks of 16 waves, a tile
+        of 16 keys per wave at a time, and as many slices as shorten a wave's walk by more
+        than the merge kernel costs, while all blocks still fit the chip at once.  More
+        pairs, and the generic kernel: blocks of 4 waves and enough slices to put about two
+        blocks on each of the 256 compute units, never more than there are pages."""
+        pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
+        n_kv_heads = self.spec.n_kv_heads
+        if self.matrix_cores:
+            # a block of 16 waves takes at most 4 query heads of a group: larger groups have
+            # several blocks per pair
+            pairs = n_seqs * n_kv_heads * ((self.group + 3) // 4)
+            if pairs <= 256:
+                tiles = (context + 15) // 16
+                best, best_cost = 1, TILE_US * ((tiles + 15) // 16)
+                slices = 2
+                while slices <= min(pages, MAX_SLICES) and pairs * 16 * slices <= WAVE_SLOTS:
+                    cost = (TILE_US * ((tiles + 16 * slices - 1) // (16 * slices)) + MERGE_US
+                            + MERGE_SLICE_US * slices)
+                    if cost < best_cost:
+                        best, best_cost = slices, cost
+                    slices *= 2
+                return best, 16
+        blocks = n_seqs * n_kv_heads
+        wanted = (512 + blocks - 1) // blocks
+        return max(1, min(wanted, pages, MAX_SLICES)), 4
+
     def forward(self, ctx, x, entry):
         spec = self.spec
         n = x.shape[0]
@@ -113,8 +191,7 @@ class Attention:
         out = ctx.buffer("attn.out", (n, spec.q_width))
         part_o = part_ml = None
         if ctx.decode:
-            splits, waves = (ctx.decode_plan(spec.n_kv_heads, self.group) if self.matrix_cores
-                             else (ctx.decode_splits(spec.n_kv_heads), 4))
+            splits, waves = self.decode_launch(ctx.n_seqs, ctx.context_bound)
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
                                     torch.float32)
@@ -127,13 +204,13 @@ class Attention:
                                           n_splits=splits, part_o=part_o, part_ml=part_ml,
                                           waves=waves, longest=meta.longest)
             else:
-                item_seq, item_row0, item_npos, n_items = meta.decode_items()
+                item_seq, item_row0, item_npos, n_items = self._items(ctx, "attention.decode_items")
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
                               scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml)
         else:
-            item_seq, item_row0, item_npos, n_items = meta.prefill_items(self.positions_per_item())
+            item_seq, item_row0, item_npos, n_items = self._items(ctx, self._items_section())
             if self.matrix_cores:
                 lib.attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos,
                                            n_items, meta.row_pos, page_table, out, spec.n_heads,

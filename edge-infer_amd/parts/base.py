@@ -49,7 +49,14 @@ class Workspace:
     buffers from the arena.  A step that asks for something else than was recorded (a
     name, an order, a larger size) is served from named buffers from there on and its
     signature is planned anew next time.  A name that is asked for again while still live
-    stands for the same storage until then, so the earlier value ends there."""
+    stands for the same storage until then, so the earlier value ends there.
+
+    `start(signature, scale)`: a signature may stand for a class of steps (prompt steps of
+    about so many rows); the recorded sizes are then multiplied by `scale`, the ratio of the
+    class's largest step to the recorded one, so that every step of the class finds room at
+    the planned places.  At most `MAX_PLANS` plans are kept; the one unused for longest goes
+    first.  `bind(name, tensor)`: requests for that name are served from the caller's tensor
+    and are not part of any plan (several workspaces can share one large buffer this way)."""
 
     MAX_PLANS = 32
 
@@ -63,23 +70,42 @@ class Workspace:
         self._events: Optional[list] = None               # recording these events
         self._cursor = 0
         self._names: Dict[int, str] = {}                  # data pointer -> name, this step
+        self._scale = 1.0
+        self._bound: Dict[str, torch.Tensor] = {}
+
+    def bind(self, name: str, tensor: Optional[torch.Tensor]) -> None:
+        """Serve requests for `name` from `tensor` (None: no longer)."""
+        if tensor is None:
+            self._bound.pop(name, None)
+        else:
+            self._bound[name] = tensor
+
+    def clear(self) -> None:
+        """Forget every plan and give all storage back."""
+        self._buffers.clear()
+        self._plans.clear()
+        self._arena = None
+        self._signature = self._layout = self._events = None
 
     # -- one step ------------------------------------------------------------
-    def start(self, signature) -> None:
+    def start(self, signature, scale: float = 1.0) -> None:
         self._signature = signature
-        self._layout = self._plans.get(signature)
+        self._layout = self._plans.pop(signature, None)
+        if self._layout is not None:
+            self._plans[signature] = self._layout         # most recently used: last
         self._events = [] if self._layout is None else None
         self._cursor = 0
+        self._scale = max(1.0, float(scale))
         self._names.clear()
 
     def finish(self) -> None:
         if self._events is not None:
-            layout = _StepLayout.from_recording(self._events)
-            if len(self._plans) >= self.MAX_PLANS:
+            layout = _StepLayout.from_recording(self._events, self._scale)
+            while len(self._plans) >= self.MAX_PLANS:
                 self._plans.pop(next(iter(self._plans)))
             self._plans[self._signature] = layout
-            if self._arena is None or self._arena.numel() < layout.plan.total_bytes:
-                self._arena = torch.empty(max(layout.plan.total_bytes, 256), dtype=torch.uint8,
+            if self._arena is None or self._arena.numel() < layout.arena.arena_bytes:
+                self._arena = torch.empty(max(layout.arena.arena_bytes, 256), dtype=torch.uint8,
                                           device=self.device)
                 for other in self._plans.values():
                     other.views.clear()               # they pointed into the old arena
@@ -100,6 +126,12 @@ class Workspace:
         count = 1
         for extent in shape:
             count *= int(extent)
+        bound = self._bound.get(name)
+        if bound is not None:
+            if bound.dtype != dtype or bound.numel() < count:
+                raise ValueError(f"the buffer bound to '{name}' holds {bound.numel()} elements of "
+                                 f"{bound.dtype}; {count} of {dtype} are wanted")
+            return bound.view(-1)[:count].view(*shape)
         layout = self._layout
         if layout is not None:
             index = self._cursor
@@ -109,7 +141,7 @@ class Workspace:
                     self._cursor = index + 1
                     view = layout.views.get(index)
                     if view is None or view.dtype != dtype or tuple(view.shape) != tuple(shape):
-                        offset = layout.plan.at(key).offset
+                        offset = layout.arena.offset(key)
                         raw = self._arena[offset:offset + count * dtype.itemsize]
                         view = raw.view(dtype).view(*shape)
                         layout.views[index] = view
@@ -152,25 +184,28 @@ class Workspace:
 class _StepLayout:
     """The recorded order of a step's requests and releases, and the plan made of it."""
 
-    def __init__(self, events, plan):
-        self.events = events      # (name, bytes, plan key) for a request, (name, None, None)
-        self.plan = plan
+    def __init__(self, events, arena):
+        self.events = events      # (name, bytes, layout key) for a request, (name, None, None)
+        self.arena = arena        # cache.workspace.ArenaLayout
         self.views: Dict[int, torch.Tensor] = {}
 
     @classmethod
-    def from_recording(cls, recorded):
+    def from_recording(cls, recorded, scale: float = 1.0):
         """recorded: (name, bytes) for each request and (name, None) for each release, in
         order; a value lives from its request to the event before its release (or before
-        the next request of its name), or to the end."""
-        from ..cache.workspace import WorkspacePlanner
-        planner = WorkspacePlanner()
-        live: Dict[str, list] = {}        # name -> [plan key, bytes, first use]
+        the next request of its name), or to the end.  Sizes are multiplied by `scale`."""
+        from ..cache.workspace import Lifetime, lay_out
+        needs = []
+        if scale > 1.0:
+            recorded = [(name, None if nbytes is None else int(-(-nbytes * scale // 1)))
+                        for name, nbytes in recorded]
+        live: Dict[str, list] = {}        # name -> [layout key, bytes, tick of the request]
         events = []
         counts: Dict[str, int] = {}
         for tick, (name, nbytes) in enumerate(recorded):
             if name in live:              # released, or asked for again: the value ends
                 key, size, first = live.pop(name)
-                planner.add_request(key, size, first, max(first, tick - 1))
+                needs.append(Lifetime(key, size, first, max(first, tick - 1)))
             if nbytes is None:
                 events.append((name, None, None))
                 continue
@@ -179,8 +214,8 @@ class _StepLayout:
             live[name] = [key, nbytes, tick]
             events.append((name, nbytes, key))
         for key, size, first in live.values():    # never released: live to the step's end
-            planner.add_request(key, size, first, len(recorded))
-        return cls(events, planner.build())
+            needs.append(Lifetime(key, size, first, len(recorded)))
+        return cls(events, lay_out(needs))
 
 
 class StepContext:
@@ -188,7 +223,7 @@ class StepContext:
     entries, the workspace and the kind of step."""
 
     def __init__(self, *, dtype, device, n_rows, n_seqs, decode, meta, cache, workspace,
-                 max_context):
+                 max_context, context_bound=None, fixed_shape=False):
         self.dtype = dtype            # storage type of activations and cache
         self.device = device
         self.n_rows = n_rows          # packed rows of this step (padding rows included)
@@ -198,6 +233,12 @@ class StepContext:
         self.cache = cache            # cache.storage.SessionCache
         self.workspace = workspace
         self.max_context = max_context  # longest sequence after this step (host value)
+        # launch shapes must hold for sequences of up to this many tokens: the longest one of
+        # the step, or more when the step is captured and replayed for longer contexts (then
+        # `fixed_shape` is set, and what depends on the true lengths is read on the device)
+        self.context_bound = max_context if context_bound is None else context_bound
+        self.fixed_shape = fixed_shape
+        self.sequences = ()             # engine.batch.SeqStep of every live sequence (host)
 
     def buffer(self, name, shape, dtype=None):
         return self.workspace.get(name, shape, self.dtype if dtype is None else dtype)

@@ -13,6 +13,10 @@ class PreNormBlock:
     parts = ("norm1", "mixer", "norm2", "ffn")
     capture_safe = True      # nothing of its own besides its parts' kernels
 
+    def members(self):
+        """The parts this block is made of, in the order in which they run."""
+        return (self.norm1, self.mixer, self.norm2, self.ffn)
+
     @classmethod
     def parameters(cls, layer_spec, hidden):
         norm_cls = lookup("norm", layer_spec.norm.kind)

@@ -53,6 +53,18 @@ class Linear:
         if dtype == torch.bfloat16 and STREAM_COPY and self.in_features % 8 == 0:
             self.packed = lib.pack_weight(self.weight)
 
+    @property
+    def capture_safe(self) -> bool:
+        """Whether a step of at most `capture_rows` rows launches nothing but this library's
+        kernels here (the library's products may record memset nodes, which are not replayed
+        reliably from a graph)."""
+        return self.dtype == torch.float32 or self.in_features % 8 == 0
+
+    @property
+    def capture_rows(self) -> int:
+        """Most rows of a step for which `capture_safe` holds."""
+        return (1 << 30) if self.dtype == torch.float32 else SKINNY_ROWS
+
     def _few_rows(self, x: torch.Tensor, out: torch.Tensor) -> None:
         if self.packed is not None:
             lib.gemm_bf16_skinny_packed(x, self.packed, self.out_features, out)
@@ -116,7 +128,10 @@ class Linear:
             if self.bias is not None:
                 lib.bias_rows(self.bias_f32, out, accumulate=True)
             return out
-        if self.in_features % 8 == 0 and rows <= max(256, SKINNY_ROWS):
+        if self.in_features % 8 == 0:
+            # any number of rows, in groups of the few-rows product with its float32 sums: a
+            # row's logits are float32 however many rows a step wants (the library's product
+            # would round them to bfloat16)
             for start in range(0, rows, SKINNY_ROWS):
                 stop = min(rows, start + SKINNY_ROWS)
                 count = stop - start
@@ -132,6 +147,7 @@ class Linear:
             if self.bias is not None:
                 lib.bias_rows(self.bias_f32, out, accumulate=True)
             return out
+        # a width that is no multiple of 8: the library's product, rounded to bfloat16
         low = ctx.buffer(out_name + ".bf16", (rows, self.out_features), torch.bfloat16)
         self._library(x, low)
         out.copy_(low)

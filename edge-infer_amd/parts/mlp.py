@@ -18,7 +18,14 @@ from .linear import Linear
 
 
 class GatedMLP:
-    capture_safe = True      # only capturable kernels, no allocation per step
+    @property
+    def capture_safe(self):
+        """Only capturable kernels and no allocation per step, as long as its products do."""
+        return self.gate_up.capture_safe and self.down.capture_safe
+
+    @property
+    def capture_rows(self):
+        return min(self.gate_up.capture_rows, self.down.capture_rows)
 
     @classmethod
     def parameters(cls, spec, hidden):

@@ -2,9 +2,12 @@
 
 angle[p, i] = float(p) * (1 / theta^(2i / d)) with the frequency and the product
 in float32, as the reference builds its table
-(runtime/include/models/qwen3_model.hpp:410-436); cosine and sine are evaluated in
-float64 from that float32 angle and rounded once.  Row p holds cos for the d/2 pairs,
-then sin; pairs are (i, i + d/2).
+(runtime/include/models/qwen3_model.hpp:410-436).  Its power is the C library's single
+precision `pow`, which works in double precision inside and rounds the result once; the
+same is done here (a float32 `pow` of another library may differ in the last bit, which
+moves the angle of position 4,000 by 2e-4).  Cosine and sine are evaluated in float64 from
+the float32 angle and rounded once.  Row p holds cos for the d/2 pairs, then sin; pairs are
+(i, i + d/2).
 """
 from __future__ import annotations
 
@@ -18,7 +21,8 @@ class RotaryTable:
         self.spec = spec
         half = spec.dim // 2
         exponent = (2.0 * torch.arange(half, dtype=torch.float32)) / float(spec.dim)
-        frequency = 1.0 / torch.pow(torch.tensor(float(spec.theta), dtype=torch.float32), exponent)
+        theta = torch.tensor(float(spec.theta), dtype=torch.float32).to(torch.float64)
+        frequency = 1.0 / torch.pow(theta, exponent.to(torch.float64)).to(torch.float32)
         position = torch.arange(spec.max_positions, dtype=torch.float32)
         angle = (position[:, None] * frequency[None, :]).to(torch.float64)
         table = torch.cat([torch.cos(angle), torch.sin(angle)], dim=1).to(torch.float32)

@@ -57,12 +57,16 @@ def linear(x, weight_out_in, bias=None):
 def rope_angles(positions, head_dim, theta):
     """angle[p, i] = float(p) * (1 / pow(theta, 2i / d)), all in float32.
 
-    runtime/include/models/qwen3_model.hpp:418-424.
+    runtime/include/models/qwen3_model.hpp:418-424: `std::pow(float, float)`, the C
+    library's single-precision power, whose result is the double-precision power rounded
+    once to float32; it is formed that way here, so that no other library's last bit of a
+    float32 power enters the angle.
     """
     half = head_dim // 2
     i = np.arange(half, dtype=np.float32)
     exponent = (np.float32(2.0) * i) / np.float32(head_dim)
-    frequency = np.float32(1.0) / np.power(np.float32(theta), exponent, dtype=np.float32)
+    power = np.power(np.float64(np.float32(theta)), exponent.astype(np.float64))
+    frequency = np.float32(1.0) / power.astype(np.float32)
     pos = np.asarray(positions, dtype=np.int64).astype(np.float32)
     angle = (pos[:, None] * frequency[None, :]).astype(np.float32)
     return torch.from_numpy(angle.astype(np.float64))

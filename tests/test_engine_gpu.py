@@ -316,10 +316,20 @@ def test_greedy_generation_through_the_entry_point(folders, oracle, name, dtype)
         assert [t for j, t in seen if j == i] == got[i]
     # the single-request call of the reference's API: max_length counts the prompt
     single = session.generate(prompts[1], max_length=len(prompts[1]) + 4, top_k=1)
-    first4 = got[1][:4]
-    if cfg["eos_token_id"] in first4:
-        first4 = first4[:first4.index(cfg["eos_token_id"])]
-    assert single == first4 or dtype == "bfloat16"
+    first4 = plain.generate(w, cfg, prompts[1], max_length=len(prompts[1]) + 4)
+    if dtype == "float32":
+        assert single == first4
+    else:
+        # alone, the request runs other launch shapes than in the batch; it may leave the
+        # plain implementation's greedy path only at a near tie, like the batch above
+        agree = 0
+        while agree < min(len(single), len(first4)) and single[agree] == first4[agree]:
+            agree += 1
+        if agree < len(first4):
+            assert agree < len(single), "the request ended early"
+            logits = plain.forward(w, cfg, prompts[1] + first4[:agree])[-1]
+            gap = (logits[first4[agree]] - logits[single[agree]]).item()
+            assert 0 <= gap <= 0.06 * logits.abs().max().item(), f"alone, step {agree}"
     assert session.generate(prompts[1], max_length=len(prompts[1])) == []
     # the end-of-sequence token ends a request and is not delivered
     if dtype == "float32":
@@ -585,21 +595,21 @@ def test_planned_workspace_gives_the_same_logits_in_less_storage(models, referen
     plans = list(session.workspace._plans.values())
     assert len(plans) == 2                                # the prompt step and the decode step
     for layout in plans:
-        plan = layout.plan
-        assert plan.reused_bytes() > 0 and plan.slot_count() < len(plan.allocations)
-        assert plan.total_bytes < plan.unaliased_bytes()
-    assert session.workspace.bytes() == max(256, max(l.plan.total_bytes for l in plans))
+        arena = layout.arena
+        assert arena.bytes_saved() > 0 and arena.regions() < len(arena)
+        assert arena.arena_bytes < arena.bytes_without_sharing()
+    assert session.workspace.bytes() == max(256, max(l.arena.arena_bytes for l in plans))
     report = session.workspace_report()
     assert report["held_bytes"] == session.workspace.bytes() and len(report["plans"]) == 2
-    assert all(p["reused_bytes"] == p["unaliased_bytes"] - p["arena_bytes"] > 0
+    assert all(p["bytes_saved"] == p["bytes_without_sharing"] - p["arena_bytes"] > 0
                for p in report["plans"].values())
     # a step that wants no logits plans none (runtime/tests/decoder_output_plan_test.cpp:11-41)
     slot = session.begin()
     for _ in range(2):
         assert session.step([(slot, prompts[0][:7], [])]).shape == (0, 381)
-    silent = [l.plan for sig, l in session.workspace._plans.items() if sig[2] == 0]
-    assert len(silent) == 1 and not any(a.name.startswith("logits") for a in silent[0].allocations)
-    assert any(a.name.startswith("logits") for a in plans[0].plan.allocations)
+    silent = [l.arena for sig, l in session.workspace._plans.items() if sig[2] == 0]
+    assert len(silent) == 1 and not any(name.startswith("logits") for name in silent[0].names())
+    assert any(name.startswith("logits") for name in plans[0].arena.names())
 
 
 def test_a_failed_step_leaves_the_session_as_it_was_and_a_failed_wait_ends_it(models, references,
@@ -646,3 +656,162 @@ def test_a_failed_step_leaves_the_session_as_it_was_and_a_failed_wait_ends_it(mo
         with pytest.raises(RuntimeError, match="unusable"):
             call()
     torch.cuda.synchronize()
+
+
+# What the bfloat16 engine may differ by from the float32 engine on eight layers of the 8B
+# shape with the real vocabulary.  Measured on an MI355X: rms 0.0174, max 0.0211, 73.5 % of
+# the logits within the reference's bound, the same top token at 90.6 % of the places (about
+# 0.2 % of rounding error per operation, ten roundings a layer, adding up like a random walk).
+DEPTH_RMS_REL = 0.02          # root-mean-square difference / root-mean-square logit
+DEPTH_MAX_REL = 0.03          # largest difference / largest logit
+DEPTH_WITHIN_REFERENCE_BOUND = 0.70   # share of logits within the reference's bound, below
+DEPTH_SAME_TOP_TOKEN = 0.85   # share of places with the same most likely token
+
+
+def test_bfloat16_against_float32_on_eight_layers_of_the_8b_shape():
+    """The two precisions of the whole engine at real width and vocabulary, deeper than
+    the tiny models: 300- and 120-token prompts, then 24 tokens one by one each.  Reported
+    and bounded: rms and largest difference, the share of logits within the reference's
+    bound |a - r| <= 0.015625 + 0.01 max(|a|, |r|) (runtime/tests/qwen3_session_test.cpp:325-326,
+    there for its two-layer test model), and how often the top token is the same.  Random
+    weights make nearly flat logits (the top two are often closer than bfloat16 resolves),
+    so equal top tokens everywhere cannot be asked for; where they differ the float32
+    engine's own margin between the two must be small."""
+    import edge_infer_amd as ei
+    cfg = ei.Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=8,
+                         num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                         intermediate_size=12288, max_position_embeddings=1024, bos_token_id=0,
+                         eos_token_id=151645, rms_norm_eps=1e-6, rope_theta=1e6,
+                         tie_word_embeddings=False)
+    prompts = [random_ids(cfg.vocab_size, 300, 41), random_ids(cfg.vocab_size, 120, 42)]
+    feed = [random_ids(cfg.vocab_size, 24, 43), random_ids(cfg.vocab_size, 24, 44)]
+
+    def run(dtype):
+        model = ei.random_model(cfg, seed=2, dtype=dtype)
+        session = ei.Session(model, max_tokens=1024, max_seqs=2)
+        slots = [session.begin(), session.begin()]
+        rows = [session.step([(s, p, list(range(len(p) - 8, len(p))))
+                              for s, p in zip(slots, prompts)])]
+        for t in range(24):
+            rows.append(session.step([(s, [f[t]], [0]) for s, f in zip(slots, feed)]))
+        assert session.graph_replays > 0
+        out = torch.cat(rows).double().cpu()
+        del session, model
+        torch.cuda.empty_cache()
+        return out
+
+    exact, low = run("float32"), run("bfloat16")
+    assert exact.shape == (16 + 48, cfg.vocab_size)
+    diff = (low - exact).abs()
+    rms = diff.pow(2).mean().sqrt().item() / exact.pow(2).mean().sqrt().item()
+    worst = diff.max().item() / exact.abs().max().item()
+    within = (diff <= 0.015625 + 0.01 * torch.maximum(low.abs(), exact.abs())).double().mean().item()
+    same = (low.argmax(-1) == exact.argmax(-1)).double().mean().item()
+    print(f"\nbfloat16 against float32, 8 layers of the 8B shape: rms {rms:.4f}, max {worst:.4f}, "
+          f"within the reference's bound {within:.4f}, same top token {same:.3f}")
+    assert rms <= DEPTH_RMS_REL and worst <= DEPTH_MAX_REL
+    assert within >= DEPTH_WITHIN_REFERENCE_BOUND and same >= DEPTH_SAME_TOP_TOKEN
+    # where the top token differs, float32 itself holds the two within bfloat16's error
+    for row in (low.argmax(-1) != exact.argmax(-1)).nonzero().flatten().tolist():
+        margin = exact[row].max() - exact[row, low[row].argmax()]
+        assert margin <= 2 * diff[row].max(), f"place {row}: margin {margin:.4f}"
+
+
+def head64_folder(root):
+    """A model whose bfloat16 steps take the matrix-core attention kernels (head size 64),
+    the decode kernel that writes the position's key and value itself included."""
+    import edge_infer_amd as ei
+    cfg = ei.Qwen3Config(vocab_size=500, hidden_size=128, num_hidden_layers=2,
+                         num_attention_heads=4, num_key_value_heads=2, head_dim=64,
+                         intermediate_size=256, max_position_embeddings=512, bos_token_id=1,
+                         eos_token_id=499, rms_norm_eps=1e-6, rope_theta=1e4,
+                         tie_word_embeddings=True)
+    return ei.write_model_folder(root / "head64", cfg, seed=5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which", ["B", "head64"])
+def test_a_step_writes_only_its_own_positions_of_the_cache(folders, tmp_path, which, dtype):
+    """The whole cache is filled with a sentinel; after every step exactly the positions
+    [old length, new length) of the stepped slots have changed, in every layer's keys and
+    values, and nothing else: not the rest of their pages, not other slots, not free pages,
+    not what a padding row of a captured step points at
+    (runtime/tests/qwen3_session_test.cpp:174-185,309-319 holds the same for its one slot)."""
+    import edge_infer_amd as ei
+    folder = folders["B"] if which == "B" else head64_folder(tmp_path)
+    model = ei.load_model(folder, dtype=dtype)
+    vocab = model.spec.vocab_size
+    session = ei.Session(model, max_tokens=12 * 64, max_seqs=4)
+    assert session.graphs
+    cache = session.cache
+    sentinel = -123.0
+    for tensor in cache.kv_k + cache.kv_v:
+        tensor.fill_(sentinel)
+
+    def stepped(entries):
+        before = [t.clone() for t in cache.kv_k + cache.kv_v]
+        old = {slot: session.length(slot) for slot, _, _ in entries}
+        session.step(entries)
+        torch.cuda.synchronize()
+        for group, pages in enumerate(cache.kv_pages):
+            expected = torch.zeros(cache.kv_k[group].shape[1:4:2], dtype=torch.bool)  # [page, 64]
+            for slot, tokens, _ in entries:
+                row = pages.row(slot)
+                for pos in range(old[slot], old[slot] + len(tokens)):
+                    expected[row[pos // 64], pos % 64] = True
+            for name, now, was in (("k", cache.kv_k[group], before[group]),
+                                   ("v", cache.kv_v[group], before[len(cache.kv_k) + group])):
+                changed = (now != was).cpu()             # [entry, page, kv head, 64, d]
+                assert torch.equal(changed.any(dim=-1).any(dim=2).any(dim=0), expected), \
+                    f"{name}: positions written differ from the step's own"
+                # ... and there every layer, head and element was written
+                written = (now != sentinel).cpu().all(dim=-1).all(dim=2).all(dim=0)
+                assert bool(written[expected].all()), name
+
+    a, b, c = (random_ids(vocab, n, 60 + i) for i, n in enumerate((130, 9, 70)))
+    sa, sb, sc = session.begin(), session.begin(), session.begin()
+    stepped([(sa, a[:100], [99]), (sb, b[:5], []), (sc, c[:64], [0, 63])])   # unequal prompts
+    stepped([(sa, a[100:101], [0]), (sb, b[5:6], [0]), (sc, c[64:65], [0])])  # eager, then captured
+    stepped([(sa, a[101:102], [0]), (sb, b[6:7], [0]), (sc, c[65:66], [0])])  # replayed, one padding row
+    assert session.graph_replays == 1
+    stepped([(sa, a[102:129], [26])])                                         # a portion of 27
+    session.end(sb)
+    sd = session.begin()                 # the slot again, with other tokens than it held
+    stepped([(sd, random_ids(vocab, 9, 99), [8]), (sc, c[66:70], [3])])
+    stepped([(sa, a[129:130], [0])])
+    session.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steady_decoding_allocates_nothing_on_the_device(folders, tmp_path, dtype):
+    """After the first steps of a batch have captured their graph, fifty more decode steps
+    (greedy sampling and the copy of the tokens included) ask the device allocator for
+    nothing (runtime/tests/qwen3_session_test.cpp:469-531 counts allocations the same way)."""
+    import edge_infer_amd as ei
+    from edge_infer_amd.sampling import Sampler, SamplingParams
+    model = ei.load_model(head64_folder(tmp_path), dtype=dtype)
+    session = ei.Session(model, max_tokens=4 * 256, max_seqs=4, max_seq_tokens=256)
+    sampler, greedy = Sampler(model.device), SamplingParams(temperature=0.0)
+    prompts = [random_ids(500, n, 80 + n) for n in (40, 3, 17)]
+    slots = [session.begin() for _ in prompts]
+    logits = session.step([(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)], copy=False)
+    tokens = sampler(logits, greedy, [], [])
+
+    def decode(count):
+        nonlocal tokens
+        for _ in range(count):
+            logits = session.step([(s, [t], [0]) for s, t in zip(slots, tokens)], copy=False)
+            tokens = sampler(logits, greedy, [], [])
+    decode(3)
+    torch.cuda.synchronize()
+    stats = torch.cuda.memory_stats()
+    before = (stats["allocation.all.allocated"], stats["segment.all.allocated"],
+              stats["allocated_bytes.all.current"], stats["reserved_bytes.all.current"])
+    replays = session.graph_replays
+    decode(50)
+    torch.cuda.synchronize()
+    stats = torch.cuda.memory_stats()
+    after = (stats["allocation.all.allocated"], stats["segment.all.allocated"],
+             stats["allocated_bytes.all.current"], stats["reserved_bytes.all.current"])
+    assert after == before, f"allocator figures moved: {before} -> {after}"
+    assert session.graph_replays == replays + 50

@@ -783,3 +783,87 @@ def test_sum_slices(lib):
     for s in range(1, 5):
         expected += slices[s]
     assert torch.equal(out, expected)
+
+
+# ---------------------------------------------------------------------------
+# The products at the widths of real checkpoints: every (out, in) of the 8B, 32B and 0.6B
+# shapes, the vocabulary of 151,936 included, at 1 to 256 rows.  The reference is a float64
+# product on the GPU (the plain implementation's `linear` is the same x . W^T).
+REAL_SHAPES = {
+    "8b": dict(H=4096, Q=4096, KV=1024, I=12288),
+    "32b": dict(H=5120, Q=8192, KV=1024, I=25600),
+    "0.6b": dict(H=1024, Q=2048, KV=1024, I=3072),
+}
+VOCABULARY = 151936
+REAL_ROWS = (1, 8, 16, 64, 256)
+
+
+def real_products(shape):
+    s = REAL_SHAPES[shape]
+    return {"qkv": (s["Q"] + 2 * s["KV"], s["H"]), "o": (s["H"], s["Q"]),
+            "gate_up": (2 * s["I"], s["H"]), "down": (s["H"], s["I"]),
+            "head": (VOCABULARY, s["H"])}
+
+
+@pytest.mark.parametrize("which", ["qkv", "o", "gate_up", "down", "head"])
+@pytest.mark.parametrize("shape", sorted(REAL_SHAPES))
+def test_gemm_bf16_skinny_at_the_widths_of_real_checkpoints(lib, shape, which):
+    N, K = real_products(shape)[which]
+    g = torch.Generator(device=DEV).manual_seed(N + K)
+    x = torch.randn(256, K, device=DEV, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, device=DEV, generator=g).to(torch.bfloat16)
+    expected = x.double() @ w.double().t()
+    packed = lib.pack_weight(w)
+    bound = 2e-6 * math.sqrt(K) * 16
+    for M in REAL_ROWS:
+        splits = lib.skinny_gemm_splits(M, N, K)
+        out = torch.full((splits, M, N), float("nan"), device=DEV)
+        lib.gemm_bf16_skinny_packed(x[:M], packed, N, out)
+        err = (out.double().sum(0) - expected[:M]).abs().max().item()
+        assert err <= bound, f"{shape} {which} {M} rows, {splits} slices: max error {err:.3e}"
+        if M in (1, 64):       # the stored layout through the other entry point
+            again = torch.full((splits, M, N), float("nan"), device=DEV)
+            lib.gemm_bf16_skinny(x[:M], w, again)
+            assert torch.equal(again, out), f"{shape} {which} {M} rows: stored layout differs"
+    if which == "gate_up":
+        # rows read as strips of 16 gate rows and their 16 up rows: the kernel's own activation
+        pairs = expected.view(256, N // 32, 2, 16)
+        gate, up = pairs[:, :, 0].reshape(256, N // 2), pairs[:, :, 1].reshape(256, N // 2)
+        wanted = gate / (1 + torch.exp(-gate)) * up
+        for M in (1, 8, 64, 256):
+            act = torch.full((M, N // 2), float("nan"), device=DEV, dtype=torch.bfloat16)
+            lib.gemm_bf16_skinny_gated(x[:M], packed, N, act, True)
+            err = (act.double() - wanted[:M]).abs().max().item()
+            assert err <= 1.2e-2 * wanted[:M].abs().max().item(), f"{shape} gated {M} rows: {err:.3e}"
+
+
+@pytest.mark.parametrize("which", ["qkv", "o", "gate_up", "down", "head"])
+@pytest.mark.parametrize("shape", sorted(REAL_SHAPES))
+def test_gemm_f32_at_the_widths_of_real_checkpoints(lib, shape, which):
+    N, K = real_products(shape)[which]
+    g = torch.Generator(device=DEV).manual_seed(N + 3 * K)
+    x = torch.randn(256, K, device=DEV, generator=g)
+    w = torch.randn(N, K, device=DEV, generator=g)
+    expected = x.double() @ w.double().t()
+    for M in REAL_ROWS:
+        out = torch.full((M, N), float("nan"), device=DEV)
+        lib.gemm_f32(x[:M], w, out)
+        err = (out.double() - expected[:M]).abs().max().item()
+        # every output is one thread's sum over k in ascending order: K roundings of 2^-24 of
+        # partial sums that grow like sqrt(k) add up to about 2^-24 K / 2.4 (one sigma)
+        assert err <= 6 * 2.0 ** -24 * K, f"{shape} {which} {M} rows: max error {err:.3e}"
+    del expected
+    torch.cuda.empty_cache()
+
+
+def test_argmax_and_sample_at_the_real_vocabulary(lib):
+    rows = 64
+    g = torch.Generator(device=DEV).manual_seed(9)
+    logits = torch.randn(rows, VOCABULARY, device=DEV, generator=g)
+    tokens = torch.empty(rows, dtype=torch.int32, device=DEV)
+    partial = torch.empty(lib.argmax_partial_size(rows, VOCABULARY), device=DEV)
+    lib.argmax(logits, tokens, None, partial)
+    assert tokens.tolist() == logits.argmax(-1).tolist()
+    static = torch.empty(rows, dtype=torch.int32, device=DEV)
+    lib.argmax_static(logits, static)
+    assert torch.equal(static, tokens)

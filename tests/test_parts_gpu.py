@@ -38,23 +38,14 @@ def random_params(spec, seed=0):
 
 def context_for(session, seqs_tokens):
     """A step context over fresh slots, without running the model."""
-    from edge_infer_amd.engine.batch import SeqStep, StepPlan
-    from edge_infer_amd.engine.session import _Context
+    from edge_infer_amd.engine.batch import SeqStep
     seqs = []
     for start, tokens in seqs_tokens:
         slot = session.begin()
         session.cache.lengths[slot] = start
         seqs.append(SeqStep(slot=slot, start=start, tokens=tokens))
     session.cache.grow([(s.slot, s.start + s.count) for s in seqs])
-    plan = StepPlan(seqs, item_sizes=session._item_sizes)
-    tables = [session.cache.page_rows(g, [s.slot for s in seqs], plan.n_seqs)
-              for g in range(len(session.cache.kv_pages))]
-    session.meta.upload(plan, tables)
-    ctx = _Context(session, dtype=session.dtype, device=session.device, n_rows=plan.n_rows,
-                   n_seqs=plan.n_seqs, decode=plan.decode, meta=session.meta, cache=session.cache,
-                   workspace=session.workspace, max_context=plan.max_context)
-    ctx.sequences = plan.seqs
-    return ctx, plan
+    return session.context_for(seqs)
 
 
 def attention_spec(**kw):
@@ -155,16 +146,10 @@ def test_attention_part(variant):
     slots = [s.slot for s in plan.seqs]
     session.cache.commit(growth)
     # the chunk: built by hand on the same slots
-    from edge_infer_amd.engine.batch import SeqStep, StepPlan
-    from edge_infer_amd.engine.session import _Context
+    from edge_infer_amd.engine.batch import SeqStep
     seqs = [SeqStep(slot=slot, start=f, tokens=[0] * 5) for slot, f in zip(slots, first)]
     session.cache.grow([(s.slot, s.start + 5) for s in seqs])
-    plan = StepPlan(seqs, item_sizes=session._item_sizes)
-    tables = [session.cache.page_rows(g, slots, plan.n_seqs) for g in range(len(session.cache.kv_pages))]
-    session.meta.upload(plan, tables)
-    ctx = _Context(session, dtype=session.dtype, device=session.device, n_rows=plan.n_rows,
-                   n_seqs=plan.n_seqs, decode=False, meta=session.meta, cache=session.cache,
-                   workspace=session.workspace, max_context=plan.max_context)
+    ctx, plan = session.context_for(seqs)
     rows, at = [], 0
     for n, f in zip(lengths, first):
         rows.append(x[at + f:at + n])
@@ -259,7 +244,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped():
         layout = session.cache.layout
         assert len(layout.kv_groups) == 2 and len(layout.state_groups) == 1
         assert layout.state_groups[0][1] == [1, 3]
-        assert session.cache.states[0].shape == (2, 3, hidden)
+        assert session.cache.states[0].shape == (2, 3 + 1, hidden)    # one spare row
 
         def oracle(ids):
             """The same model, whole sequence, float64."""
