@@ -10,6 +10,11 @@ plus generated tokens and is clipped to the capacity; a request whose limit does
 not exceed its prompt produces nothing; the first token is drawn from the last
 prompt row; a stop token ends the request and is not delivered.
 
+A batch's prompts run in one step while they have at most `prompt_rows` tokens together;
+beyond that they run in several steps of at most that many rows (whole prompts while they
+fit, then portions), so that the step workspace, which grows with the rows of a step, stays
+bounded however many long prompts start together.
+
 The loop decides; it computes nothing.  It talks to a session through `begin`,
 `step`, `end`, `capacity`, `free_tokens`, `max_batch` and to a sampler through one
 call, so its decisions are tested without a GPU.
@@ -59,10 +64,35 @@ def plan_batches(requests: Sequence[Request], max_batch: int, free_tokens: int) 
     return batches
 
 
+PROMPT_ROWS = 8192      # most rows of one prompt step
+
+
+def prompt_steps(batch: Sequence[Request], budget: int):
+    """The prompt steps of a batch: lists of (request, first token, tokens, whether the
+    prompt ends here), each list at most `budget` tokens, prompts in order."""
+    if budget < 1:
+        raise ValueError("a prompt step needs room for at least one row")
+    steps, current, room = [], [], budget
+    for request in batch:
+        done = 0
+        while done < len(request.prompt):
+            take = min(room, len(request.prompt) - done)
+            current.append((request, done, take, done + take == len(request.prompt)))
+            done += take
+            room -= take
+            if room == 0:
+                steps.append(current)
+                current, room = [], budget
+    if current:
+        steps.append(current)
+    return steps
+
+
 def generate(session, sampler, prompts: Sequence[Sequence[int]], *, vocab_size: int,
              max_length=None, max_new_tokens=None, params: Optional[SamplingParams] = None,
              stop_ids: Sequence[int] = (), callback: Optional[Callable[[int, int], None]] = None,
-             max_batch: Optional[int] = None, first_stream: int = 0) -> List[List[int]]:
+             max_batch: Optional[int] = None, first_stream: int = 0,
+             prompt_rows: int = PROMPT_ROWS) -> List[List[int]]:
     """Generate for every prompt; returns the new tokens of each, in order.
 
     max_length (an int or one per prompt) counts prompt plus generated tokens;
@@ -107,7 +137,8 @@ def generate(session, sampler, prompts: Sequence[Sequence[int]], *, vocab_size: 
 
     batch_limit = session.max_batch if max_batch is None else min(max_batch, session.max_batch)
     for batch in plan_batches(requests, batch_limit, session.free_tokens()):
-        _run_batch(session, sampler, batch, params, stop, vocab_size, callback, requests)
+        _run_batch(session, sampler, batch, params, stop, vocab_size, callback, requests,
+                   prompt_rows)
     return [request.output for request in requests]
 
 
@@ -127,12 +158,28 @@ def _deliver(request: Request, token: int, stop, vocab_size, callback, index) ->
         request.done, request.finish_reason = True, "length"
 
 
-def _run_batch(session, sampler, batch, params, stop, vocab_size, callback, all_requests) -> None:
+def _prefill(session, batch, prompt_rows):
+    """Run the prompts; logits [len(batch), vocab] at each prompt's last token."""
+    steps = prompt_steps(batch, prompt_rows)
+    if len(steps) == 1:
+        return session.step([(r.slot, r.prompt, [len(r.prompt) - 1]) for r in batch], copy=False)
+    import torch
+    rows = []
+    for step in steps:
+        logits = session.step([(r.slot, r.prompt[first:first + count], [count - 1] if last else [])
+                               for r, first, count, last in step], copy=False)
+        if logits.shape[0]:
+            rows.append(logits.clone())     # the next step overwrites what this one returned
+    return torch.cat(rows)                  # prompts end in the order of the batch
+
+
+def _run_batch(session, sampler, batch, params, stop, vocab_size, callback, all_requests,
+               prompt_rows=PROMPT_ROWS) -> None:
     index_of = {id(r): i for i, r in enumerate(all_requests)}
     try:
         for request in batch:
             request.slot = session.begin()
-        logits = session.step([(r.slot, r.prompt, [len(r.prompt) - 1]) for r in batch], copy=False)
+        logits = _prefill(session, batch, prompt_rows)
         active = list(batch)
         while True:
             tokens = sampler(logits, params, [r.stream for r in active],

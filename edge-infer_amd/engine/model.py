@@ -199,7 +199,7 @@ class DecoderModel:
     def forward(self, ctx) -> torch.Tensor:
         """Run the rows of `ctx`; float32 logits [wanted rows, vocab].  The step's buffers
         are planned by the workspace per shape of step: rows, sequences, wanted rows, kind,
-        and the context bound that fixes the launch shape of decode attention."""
+        and, for a captured step, the context bound that fixes the parts' launch shapes."""
         workspace = ctx.workspace
         workspace.start(*workspace_class(ctx))
         try:

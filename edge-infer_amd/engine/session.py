@@ -171,9 +171,11 @@ class Session:
     # -- generation ----------------------------------------------------------
     def generate_batch(self, prompts, *, max_length=None, max_new_tokens=None, temperature=1.0,
                        top_p=0.9, top_k=1, seed=None, stop_ids=None, callback=None,
-                       max_batch=None, first_stream=None):
+                       max_batch=None, first_stream=None, prompt_rows=None):
         """New tokens for every prompt (lists of ints), served in batches of prompts
-        that start together.  `callback(index, token)` sees each delivered token."""
+        that start together.  `callback(index, token)` sees each delivered token.
+        `prompt_rows`: most tokens of one prompt step (default 8,192; more prompt tokens than
+        that run in several steps)."""
         from ..sampling.params import SamplingParams
         from ..sampling.sampler import Sampler
         from .generate import generate
@@ -194,7 +196,8 @@ class Session:
             return generate(self, self._sampler, prompts, vocab_size=spec.vocab_size,
                             max_length=max_length, max_new_tokens=max_new_tokens, params=params,
                             stop_ids=stop_ids, callback=callback, max_batch=max_batch,
-                            first_stream=first_stream)
+                            first_stream=first_stream,
+                            **({} if prompt_rows is None else {"prompt_rows": int(prompt_rows)}))
         finally:
             self._busy = False
 

@@ -815,3 +815,35 @@ def test_steady_decoding_allocates_nothing_on_the_device(folders, tmp_path, dtyp
              stats["allocated_bytes.all.current"], stats["reserved_bytes.all.current"])
     assert after == before, f"allocator figures moved: {before} -> {after}"
     assert session.graph_replays == replays + 50
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_prompts_in_portions_give_the_logits_of_whole_prompts(tmp_path, dtype):
+    """The generation loop's prompt steps under a row budget of 64: a prompt cut at 64 and
+    128, a portion of 2 tokens, requests that are left out of a step, at head size 64 (the
+    matrix-core kernels in bfloat16), against whole prompts in the plain implementation."""
+    import edge_infer_amd as ei
+    from edge_infer_amd.engine.generate import Request, _prefill, prompt_steps
+    folder = head64_folder(tmp_path)
+    cfg, w = plain.read_folder(folder)
+    prompts = [random_ids(500, n, 30 + n) for n in (70, 5, 130, 33, 52)]
+    session = ei.Session(ei.load_model(folder, dtype=dtype), max_tokens=8 * 192, max_seqs=5)
+    requests = [Request(prompt=p, limit=200, stream=i) for i, p in enumerate(prompts)]
+    portions = [[(r.stream, first, count) for r, first, count, _ in step]
+                for step in prompt_steps(requests, 64)]
+    assert portions == [[(0, 0, 64)], [(0, 64, 6), (1, 0, 5), (2, 0, 53)], [(2, 53, 64)],
+                        [(2, 117, 13), (3, 0, 33), (4, 0, 18)], [(4, 18, 34)]]
+    for request in requests:
+        request.slot = session.begin()
+    logits = _prefill(session, requests, 64)
+    expected = torch.stack([plain.forward(w, cfg, p)[-1] for p in prompts])
+    assert_close(dtype, logits, expected, f"{dtype} prompts in portions")
+    assert [session.length(r.slot) for r in requests] == [70, 5, 130, 33, 52]
+    # and through the whole loop: the same tokens as with one prompt step
+    session.reset()
+    few = session.generate_batch(prompts, max_new_tokens=5, temperature=0.0, stop_ids=(),
+                                 prompt_rows=64)
+    if dtype == "float32":
+        assert few == [plain.generate(w, cfg, p, max_length=len(p) + 5, stop_ids=set())
+                       for p in prompts]
+    assert [len(tokens) for tokens in few] == [5] * 5

@@ -47,7 +47,7 @@ class ScriptedSession:
                 row[(tokens[w] + 1) % VOCAB] = 5.0
                 rows.append(row)
             self.live[slot].extend(tokens)
-        return torch.stack(rows)
+        return torch.stack(rows) if rows else torch.zeros(0, VOCAB)
 
 
 def argmax_sampler(logits, params, streams, counters):
@@ -155,3 +155,30 @@ def test_sampling_params_rules():
         SamplingParams(temperature=float("nan")).validate(10)
     with pytest.raises(ValueError, match="1024"):
         SamplingParams(temperature=1.0, top_k=2000).validate(5000)
+
+
+def test_prompts_beyond_the_row_budget_run_in_portions():
+    """Prompts of 5, 1, 7 and 2 tokens with room for 4 rows a step: whole prompts while they
+    fit, then portions; only the step that holds a prompt's last token wants its logits, and
+    the first tokens are drawn for the requests in their own order."""
+    from edge_infer_amd.engine.generate import prompt_steps
+    prompts = [[1, 2, 3, 4, 5], [10], [20, 21, 22, 23, 24, 25, 26], [28, 29]]
+    s = ScriptedSession(max_batch=4)
+    out = run(s, prompts, max_new_tokens=2, prompt_rows=4)
+    assert out == [[6, 7], [11, 12], [27, 28], [30, 31]]
+    prefill = s.steps[:4]
+    assert [[(len(t), w) for _, t, w in step] for step in prefill] == [
+        [(4, [])], [(1, [0]), (1, [0]), (2, [])], [(4, [])], [(1, [0]), (2, [1])]]
+    assert [t for step in prefill for slot, t, _ in step if slot == 2] == \
+        [[20, 21], [22, 23, 24, 25], [26]]
+    assert all(len(t) == 1 for step in s.steps[4:] for _, t, _ in step) and len(s.steps) == 5
+    # room for everything: one step, as before
+    s = ScriptedSession(max_batch=4)
+    assert run(s, prompts, max_new_tokens=1, prompt_rows=15) == [[6], [11], [27], [30]]
+    assert len(s.steps) == 1
+    requests = [Request(prompt=p, limit=99, stream=i) for i, p in enumerate(prompts)]
+    assert [[(r.stream, first, count, last) for r, first, count, last in step]
+            for step in prompt_steps(requests, 6)] == [
+        [(0, 0, 5, True), (1, 0, 1, True)], [(2, 0, 6, False)], [(2, 6, 1, True), (3, 0, 2, True)]]
+    with pytest.raises(ValueError):
+        prompt_steps(requests, 0)
