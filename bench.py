@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
                     [--shape 8b|0.6b|32b] [--only decode|prefill|generate] [--prompt P]
+                    [--with-32b] [--peaks]
 
 Prints one JSON line.  `value` is decoded tokens per second at the given batch after
 512-token prompts (one step = one decode step of the whole batch: the model, greedy
@@ -12,8 +13,12 @@ headline batch without HIP graphs.
 `--only generate` times the generation loop instead: a batch of prompts with lengths
 uniform in [64, 2048] that start together, then `--new-tokens` greedy tokens each (the
 workload named for the 0.6B shape, with `--shape 0.6b --batch 32 --context 8192`).
+`points` also hold the generation workload of the 0.6B shape (its decode step and its
+prompt step) and, with `--with-32b`, decode at batch 1 and 16 and the prefill of the 32B shape.
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
-ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s.
+ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
+a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
+roofline and prefill fractions are given against those as well (`frac_measured`).
 """
 import argparse
 import json
@@ -73,38 +78,43 @@ def synthetic_prompts(cfg, batch, length, seed):
     return torch.randint(0, cfg.vocab_size, (batch, length), generator=g).tolist()
 
 
-def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True):
-    """(ms per step, mean context during the timed steps)."""
+def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True, context=CONTEXT):
+    """(mean ms per step, mean context during the timed steps, median ms per step)."""
     import torch
     import edge_infer_amd as ei
     from edge_infer_amd.sampling import Sampler, SamplingParams
-    session = ei.Session(model, max_tokens=batch * CONTEXT, max_seqs=batch,
-                         max_seq_tokens=CONTEXT, graphs=graphs)
+    session = ei.Session(model, max_tokens=batch * context, max_seqs=batch,
+                         max_seq_tokens=context, graphs=graphs)
     sampler = Sampler(model.device)
     greedy = SamplingParams(temperature=0.0)
     prompts = synthetic_prompts(cfg, batch, prompt, seed=100 + batch)
     slots = [session.begin() for _ in range(batch)]
     logits = session.step([(s, p, [prompt - 1]) for s, p in zip(slots, prompts)], copy=False)
     tokens = sampler(logits, greedy, [], [])
+    stamps = []
 
     def run(count):
         nonlocal tokens
         for _ in range(count):
             logits = session.step([(s, [t], [0]) for s, t in zip(slots, tokens)], copy=False)
-            tokens = sampler(logits, greedy, [], [])
+            tokens = sampler(logits, greedy, [], [])     # (fetches the tokens: the step is over)
+            stamps.append(time.perf_counter())
 
     run(warmup)
     torch.cuda.synchronize()
+    stamps.clear()
     started = time.perf_counter()
     run(steps)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - started
-    context = prompt + warmup + (steps + 1) / 2
+    each = sorted(b - a for a, b in zip([started] + stamps[:-1], stamps))
+    median = each[len(each) // 2] if len(each) % 2 else (each[len(each) // 2 - 1] + each[len(each) // 2]) / 2
+    mean_context = prompt + warmup + (steps + 1) / 2
     for s in slots:
         session.end(s)
     del session
     torch.cuda.empty_cache()
-    return 1000.0 * elapsed / steps, context
+    return 1000.0 * elapsed / steps, mean_context, 1000.0 * median
 
 
 def measure_prefill(model, cfg, repeats=3):
@@ -159,6 +169,70 @@ def measure_generate(model, cfg, batch, context, new_tokens, repeats=2):
     return total, prompt_s, sum(lengths), sum(len(o) for o in out)
 
 
+def measure_peaks():
+    """What a plain read kernel streams (GB/s) and a loop of matrix-core products computes
+    (TFLOP/s, bfloat16) on this GPU: the best of a few runs each."""
+    import torch
+    from edge_infer_amd.csrc import lib
+    device = torch.device("cuda")
+    data = torch.empty(4 * 1024 ** 3, dtype=torch.uint8, device=device)
+    data.fill_(1)
+    sink = torch.zeros(4, dtype=torch.int32, device=device)
+    fsink = torch.zeros(4, dtype=torch.float32, device=device)
+
+    def best(launch, repeats=5):
+        times = []
+        for _ in range(repeats + 1):
+            begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            begin.record()
+            launch()
+            end.record()
+            end.synchronize()
+            times.append(begin.elapsed_time(end) * 1e-3)
+        return min(times[1:])
+    read_s = min(best(lambda: lib.stream_read(data, sink, blocks)) for blocks in (2048, 4096, 8192))
+    iters, blocks = 20000, 256 * 8
+    mfma_s = min(best(lambda: lib.mfma_loop(iters, blocks, fsink, wide)) for wide in (False, True))
+    flops = lib.MFMA_LOOP_FLOPS * iters * blocks * 4
+    del data
+    torch.cuda.empty_cache()
+    return {"hbm_read_GBs": round(data_bytes_of(4) / read_s / 1e9, 1),
+            "mfma_bf16_TFLOPs": round(flops / mfma_s / 1e12, 1)}
+
+
+def data_bytes_of(gib):
+    return gib * 1024 ** 3
+
+
+def other_shape_points(args):
+    """Decode and prefill figures of the other shapes, as flat numbers for `points`."""
+    import torch
+    import edge_infer_amd as ei
+    points = {}
+    cfg = model_config("0.6b", 0)
+    model = ei.random_model(cfg, seed=3, dtype=args.dtype)
+    total, prompt_s, prompt_tokens, new = measure_generate(model, cfg, 32, 8192, 256, repeats=1)
+    points["gen_0.6b_b32_new_tokens_per_s"] = round(new / total, 1)
+    points["gen_0.6b_b32_ms_per_decode_step"] = round(1e3 * (total - prompt_s) / 255, 4)
+    points["gen_0.6b_b32_prompt_tokens_per_s"] = round(prompt_tokens / prompt_s, 1)
+    del model
+    torch.cuda.empty_cache()
+    if args.with_32b:
+        cfg = model_config("32b", 0)
+        model = ei.random_model(cfg, seed=4, dtype=args.dtype)
+        for batch in (1, 16):
+            ms, _, median = measure_decode(model, cfg, batch, 16, 4)
+            points[f"32b_decode_b{batch}"] = round(batch * 1000.0 / ms, 1)
+            points[f"32b_decode_b{batch}_ms_median"] = round(median, 4)
+        ms = measure_prefill(model, cfg, repeats=2)
+        points["32b_prefill_tokens_per_s"] = round(PREFILL_TOKENS * 1000.0 / ms, 1)
+        points["32b_prefill_frac"] = round(prefill_flops(cfg, PREFILL_TOKENS) / (ms * 1e-3)
+                                           / (PEAK_TFLOPS[args.dtype] * 1e12), 4)
+        del model
+        torch.cuda.empty_cache()
+    return points
+
+
 def main():
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -179,6 +253,10 @@ def main():
                         help="tokens a sequence may hold (with --only generate)")
     parser.add_argument("--new-tokens", type=int, default=256,
                         help="tokens generated for each prompt (with --only generate)")
+    parser.add_argument("--with-32b", action="store_true",
+                        help="also measure the 32B shape (decode at batch 1 and 16, prefill)")
+    parser.add_argument("--peaks", action="store_true",
+                        help="measure the read and matrix-core yardsticks only")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
@@ -186,6 +264,10 @@ def main():
 
     import torch
     import edge_infer_amd as ei
+    if args.peaks:
+        print(json.dumps({"only": "peaks", **measure_peaks(),
+                          "published": {"hbm_GBs": HBM_PEAK_GBS, "mfma_bf16_TFLOPs": PEAK_TFLOPS["bfloat16"]}}))
+        return 0
     cfg = model_config(args.shape, args.layers)
     full_layers = SHAPES[args.shape][0]
     model = ei.random_model(cfg, seed=2, dtype=args.dtype)
@@ -193,11 +275,11 @@ def main():
     itemsize = 2 if args.dtype == "bfloat16" else 4
 
     if args.only == "decode":
-        ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup,
-                                          args.prompt)
+        ms_step, context, median = measure_decode(model, cfg, args.batch, args.steps, args.warmup,
+                                                  args.prompt, context=max(CONTEXT, args.context))
         rate = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9
         print(json.dumps({"only": "decode", "shape": args.shape, "batch": args.batch,
-                          "ms_per_step": round(ms_step, 4),
+                          "ms_per_step": round(ms_step, 4), "ms_per_step_median": round(median, 4),
                           "tokens_per_s": round(args.batch * 1000.0 / ms_step, 1),
                           "context": round(context), "GB/s": round(rate, 1)}))
         return 0
@@ -220,7 +302,7 @@ def main():
                           "ms": round(prefill_ms, 3),
                           "TFLOP/s": round(flops / (prefill_ms * 1e-3) / 1e12, 1)}))
         return 0
-    ms_step, context = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
+    ms_step, context, median_step = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
     value = args.batch * 1000.0 / ms_step
     achieved = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9
     prefill_ms = measure_prefill(model, cfg)
@@ -228,18 +310,24 @@ def main():
     points = {}
     if not args.skip_points:
         for name, batch in (("decode_b1", 1), ("decode_b64", 64)):
-            ms, _ = measure_decode(model, cfg, batch, max(8, args.steps // 2), args.warmup)
+            ms, _, _ = measure_decode(model, cfg, batch, max(8, args.steps // 2), args.warmup)
             points[name] = round(batch * 1000.0 / ms, 1)
         # the headline batch with every kernel launched by the host instead of from a HIP graph
-        ms, _ = measure_decode(model, cfg, args.batch, max(8, args.steps // 2), args.warmup,
-                               graphs=False)
+        ms, _, _ = measure_decode(model, cfg, args.batch, max(8, args.steps // 2), args.warmup,
+                                  graphs=False)
         points[f"decode_b{args.batch}_eager"] = round(args.batch * 1000.0 / ms, 1)
+    peaks = measure_peaks()
+    if not args.skip_points and args.shape == "8b":
+        del model
+        torch.cuda.empty_cache()
+        points.update(other_shape_points(args))
     from edge_infer_amd.csrc import lib
     record = {
         "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch} after "
                   f"{PROMPT}-token prompts",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True,
+        "warmup": args.warmup, "ms_per_step": round(ms_step, 4),
+        "ms_per_step_median": round(median_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
         "data": "synthetic token ids, seeded random weights N(0, 0.02)",
@@ -256,9 +344,14 @@ def main():
         },
         "prefill": {"value": round(PREFILL_TOKENS * 1000.0 / prefill_ms, 1),
                     "tokens": PREFILL_TOKENS, "ms": round(prefill_ms, 3),
-                    "frac": round(flops / (prefill_ms * 1e-3) / (PEAK_TFLOPS[args.dtype] * 1e12), 4)},
+                    "frac": round(flops / (prefill_ms * 1e-3) / (PEAK_TFLOPS[args.dtype] * 1e12), 4),
+                    "frac_measured": round(flops / (prefill_ms * 1e-3)
+                                           / (peaks["mfma_bf16_TFLOPs"] * 1e12), 4)
+                    if args.dtype == "bfloat16" else None},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "frac_measured": round(achieved / peaks["hbm_read_GBs"], 4)},
+        "measured_peaks": peaks,
         "points": points,
     }
     print(json.dumps(record))

@@ -118,18 +118,33 @@ class SequencePages:
         self.pool = pool
         self.window = window
         self._pages: Dict[int, List[int]] = {}
+        self._version: Dict[int, int] = {}     # counts the changes of a slot's page list
+        self._changes = 0
         self.n_slots = n_slots
 
     def open(self, slot: int) -> None:
         if slot in self._pages:
             raise RuntimeError(f"slot {slot} opened twice")
         self._pages[slot] = []
+        self._touch(slot)
+
+    def _touch(self, slot: int) -> None:
+        self._changes += 1
+        self._version[slot] = self._changes
+
+    def version(self, slot: int) -> int:
+        """A number that is new whenever the slot's page list has changed (no two states of
+        any slot share one, so it also tells a reopened slot from its earlier life)."""
+        return self._version[slot]
 
     def pages_needed(self, slot: int, new_length: int) -> int:
         return max(0, pages_for(new_length) - len(self._pages[slot]))
 
     def grow(self, slot: int, new_length: int) -> None:
-        self._pages[slot].extend(self.pool.alloc(self.pages_needed(slot, new_length)))
+        need = self.pages_needed(slot, new_length)
+        if need:
+            self._pages[slot].extend(self.pool.alloc(need))
+            self._touch(slot)
 
     def trim(self, slot: int, length: int) -> None:
         """Give back pages wholly before the window of the next query."""
@@ -142,10 +157,13 @@ class SequencePages:
             if page >= 0 and (index + 1) * PAGE_TOKENS - 1 < first_visible:
                 dead.append(page)
                 pages[index] = -1
-        self.pool.free(dead)
+        if dead:
+            self.pool.free(dead)
+            self._touch(slot)
 
     def close(self, slot: int) -> None:
         self.pool.free([p for p in self._pages.pop(slot) if p >= 0])
+        self._version.pop(slot, None)
 
     def row(self, slot: int) -> Sequence[int]:
         return self._pages[slot]

@@ -79,6 +79,7 @@ class SessionCache:
             shape = (len(entries), self.n_pages, request.n_kv_heads, PAGE_TOKENS, request.head_dim)
             self.kv_k.append(torch.empty(shape, dtype=dtype, device=device))
             self.kv_v.append(torch.empty(shape, dtype=dtype, device=device))
+        self._page_mirror: List[Dict[int, tuple]] = [{} for _ in self.kv_pages]
         self.states: List[torch.Tensor] = []
         self._state_copies: List[torch.Tensor] = []     # [slots, entries, *shape], see save_states
         for request, entries in layout.state_groups:
@@ -169,10 +170,16 @@ class SessionCache:
         """int32 [n_rows, table_width]: logical page -> physical page (-1: none) for
         the given slots; rows beyond them are padding."""
         table = np.full((n_rows, self.table_width), -1, dtype=np.int32)
-        pages = self.kv_pages[group]
+        pages, mirror = self.kv_pages[group], self._page_mirror[group]
         for i, slot in enumerate(slots):
             row = pages.row(slot)
-            table[i, :len(row)] = row
+            # a slot's row is kept as an array and refreshed only when its pages change (they
+            # change when the sequence passes a page boundary, not with every token)
+            version = pages.version(slot)
+            kept = mirror.get(slot)
+            if kept is None or kept[0] != version:
+                kept = mirror[slot] = (version, np.asarray(row, dtype=np.int32))
+            table[i, :kept[1].size] = kept[1]
         return table
 
     def bytes(self) -> int:

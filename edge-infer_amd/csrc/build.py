@@ -20,7 +20,7 @@ from pathlib import Path
 
 SOURCE_DIR = Path(__file__).resolve().parent
 LIBRARIES = ("rowwise", "rope_store", "attention_generic", "attention_mfma", "gemm_f32",
-             "gemm_bf16", "sampling")
+             "gemm_bf16", "sampling", "peaks")
 ARCH = "gfx950"
 # packed-fp32 instructions are switched off for every device compilation
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",

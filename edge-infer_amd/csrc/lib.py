@@ -80,6 +80,10 @@ _SIGNATURES = {
                       c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
         "ei_sample_scratch_size": [c_int, c_int],
     },
+    "peaks": {
+        "ei_stream_read": [c_void_p, c_longlong, c_int, c_void_p, c_void_p],
+        "ei_mfma_loop": [c_int, c_int, c_int, c_void_p, c_void_p],
+    },
 }
 
 _loaded: Dict[str, ctypes.CDLL] = {}
@@ -589,3 +593,25 @@ def gemm_bf16_skinny_gated(x: torch.Tensor, w: torch.Tensor, n: int, act: torch.
                                            _gpu(act, "act", torch.bfloat16), m, n, k, int(packed),
                                            _stream())
     _check(lib, status, "gemm_bf16_skinny_gated")
+
+
+# ---------------------------------------------------------------------------
+def stream_read(data: torch.Tensor, sink: torch.Tensor, blocks: int = 4096) -> None:
+    """Read every byte of `data` once with a plain kernel (a yardstick for memory-bound steps)."""
+    lib = library("peaks")
+    nbytes = data.numel() * data.element_size()
+    status = lib.ei_stream_read(_gpu(data, "data"), nbytes - nbytes % 16, int(blocks),
+                                _gpu(sink, "sink", torch.int32), _stream())
+    _check(lib, status, "stream_read")
+
+
+MFMA_LOOP_FLOPS = 8 * 16 * 16 * 32 * 2      # per wave and iteration of `mfma_loop`
+
+
+def mfma_loop(iters: int, blocks: int, sink: torch.Tensor, wide: bool = False) -> None:
+    """`blocks` x 4 waves multiply bfloat16 tiles on registers: `iters` rounds of 8 products of
+    16x16x32, or (wide) of 4 products of 32x32x16; `MFMA_LOOP_FLOPS` a wave and round."""
+    lib = library("peaks")
+    status = lib.ei_mfma_loop(int(iters), int(blocks), int(wide),
+                              _gpu(sink, "sink", torch.float32), _stream())
+    _check(lib, status, "mfma_loop")

@@ -85,18 +85,35 @@ class StepPlan:
         self.seq_start = np.zeros(self.n_seqs, dtype=np.int32)
         self.seq_count = np.zeros(self.n_seqs, dtype=np.int32)
         want_rows: List[int] = []
-        for index, seq in enumerate(seqs):
-            rows = slice(seq.row0, seq.row0 + seq.count)
-            self.tokens[rows] = np.asarray(seq.tokens, dtype=np.int64)
-            self.row_pos[rows] = np.arange(seq.start, seq.start + seq.count)
-            self.row_seq[rows] = index
-            self.seq_slot[index] = seq.slot
-            self.seq_start[index] = seq.start
-            self.seq_count[index] = seq.count
-            for w in seq.want:
-                if not 0 <= w < seq.count:
-                    raise ValueError(f"wanted place {w} is outside the {seq.count} tokens given")
-                want_rows.append(seq.row0 + w)
+        if self.decode:                  # one row a sequence: whole arrays at once
+            live = len(seqs)
+            starts = np.fromiter((seq.start for seq in seqs), dtype=np.int32, count=live)
+            self.tokens[:live] = np.fromiter((seq.tokens[0] for seq in seqs), dtype=np.int64,
+                                             count=live)
+            self.row_pos[:live] = starts
+            self.row_seq[:live] = np.arange(live, dtype=np.int32)
+            self.seq_slot[:live] = np.fromiter((seq.slot for seq in seqs), dtype=np.int32,
+                                               count=live)
+            self.seq_start[:live] = starts
+            self.seq_count[:live] = 1
+            for seq in seqs:
+                for w in seq.want:
+                    if w != 0:
+                        raise ValueError(f"wanted place {w} is outside the 1 token given")
+                    want_rows.append(seq.row0)
+        else:
+            for index, seq in enumerate(seqs):
+                rows = slice(seq.row0, seq.row0 + seq.count)
+                self.tokens[rows] = np.asarray(seq.tokens, dtype=np.int64)
+                self.row_pos[rows] = np.arange(seq.start, seq.start + seq.count)
+                self.row_seq[rows] = index
+                self.seq_slot[index] = seq.slot
+                self.seq_start[index] = seq.start
+                self.seq_count[index] = seq.count
+                for w in seq.want:
+                    if not 0 <= w < seq.count:
+                        raise ValueError(f"wanted place {w} is outside the {seq.count} tokens given")
+                    want_rows.append(seq.row0 + w)
         self.n_want_live = len(want_rows)
         if self.padded:
             # a fixed-size decode batch asks for every row; dead rows are marked -1
@@ -141,9 +158,16 @@ class DeviceMeta:
         self.n_seqs = 0
         self.n_want = 0
         self._copied = None
+        self._shape = None            # (name, size) of every section of the last upload
+        self._offsets: List[int] = []
+        self._total = 0
+        # counts the layouts this buffer has had: while it stays the same, every view is
+        # where it was (what a captured step relies on)
+        self.generation = 0
 
     def _reserve(self, count: int) -> None:
         if self._device_buffer is None or self._device_buffer.numel() < count:
+            self._copied = None
             size = max(count, 1024)
             self._device_buffer = torch.empty(size, dtype=torch.int32, device=self.device)
             pin = self.device is not None and torch.device(self.device).type == "cuda"
@@ -156,21 +180,28 @@ class DeviceMeta:
 
     def upload(self, plan: StepPlan, page_tables: Sequence[np.ndarray]) -> None:
         sections = plan.sections(page_tables)
-        offsets, total = [], 0
-        for _, array in sections:
-            offsets.append(total)
-            total += (array.size + 3) // 4 * 4
-        self._reserve(total)
+        shape = tuple((name, array.size) for name, array in sections)
+        if shape != self._shape or self._device_buffer is None:
+            # another set of sections: lay them out anew (each starts at a multiple of 4 words)
+            offsets, total = [], 0
+            for _, size in shape:
+                offsets.append(total)
+                total += (size + 3) // 4 * 4
+            self._reserve(total)
+            self._views = {name: self._device_buffer[offset:offset + size]
+                           for (name, size), offset in zip(shape, offsets)}
+            self._shape, self._offsets, self._total = shape, offsets, total
+            self.generation += 1
         if self._copied is not None:
             self._copied.synchronize()   # the last upload has left the staging buffer
         host = self._host_buffer.numpy()
-        self._views = {}
-        for (name, array), offset in zip(sections, offsets):
-            host[offset:offset + array.size] = array
-            self._views[name] = self._device_buffer[offset:offset + array.size]
+        for (_, array), offset in zip(sections, self._offsets):
+            host[offset:offset + array.size] = array.reshape(-1)
+        total = self._total
         self._device_buffer[:total].copy_(self._host_buffer[:total], non_blocking=True)
         if self._device_buffer.is_cuda:
-            self._copied = torch.cuda.Event()
+            if self._copied is None:
+                self._copied = torch.cuda.Event()
             self._copied.record()
         self._table_widths = [table.shape[1] for table in page_tables]
         self.n_seqs = plan.n_seqs
@@ -184,13 +215,6 @@ class DeviceMeta:
         except KeyError:
             raise KeyError(f"the step's metadata holds no section '{name}'; "
                            f"it holds {sorted(self._views)}") from None
-
-    def layout(self):
-        """(name, offset, size) of every section: two uploads with the same layout leave
-        every view where it was (what a captured step relies on)."""
-        base = self._device_buffer.data_ptr()
-        return tuple((name, (view.data_ptr() - base) // 4, view.numel())
-                     for name, view in self._views.items())
 
     longest = property(lambda self: self.section("longest"))
     tokens = property(lambda self: self.section("tokens"))

@@ -150,13 +150,31 @@ class DecoderModel:
                 limit = min(limit, table.max_positions)
         return limit
 
+    def _planners(self):
+        """The parts that plan metadata sections of their own, each kind once: parts that
+        would plan the same sections say so with an equal `plan_key` (36 attention layers of
+        one shape plan one work list, not 36)."""
+        found = getattr(self, "_planner_list", None)
+        if found is None:
+            found, seen = [], set()
+            for layer in self.layers:
+                for part in (layer, *members_of(layer)):
+                    if not hasattr(part, "plan_step"):
+                        continue
+                    key = getattr(part, "plan_key", None)
+                    if key is not None:
+                        if key in seen:
+                            continue
+                        seen.add(key)
+                    found.append(part)
+            self._planner_list = found
+        return found
+
     def plan_step(self, plan) -> None:
-        """Let every part add the metadata sections it plans for itself (work items of its
-        kernels and the like) to the step plan; the engine only carries them."""
-        for layer in self.layers:
-            for part in (layer, *members_of(layer)):
-                if hasattr(part, "plan_step"):
-                    plan.add_sections(part.plan_step(plan))
+        """Let the parts add the metadata sections they plan for themselves (work items of
+        their kernels and the like) to the step plan; the engine only carries them."""
+        for part in self._planners():
+            plan.add_sections(part.plan_step(plan))
 
     def capture_safe(self) -> bool:
         """Whether a decode step may be captured in a HIP graph: the final norm, the head,

@@ -230,11 +230,12 @@ class Session:
             if not tokens:
                 raise ValueError("an entry brings at least one token")
             for index, token in enumerate(tokens):
-                if not isinstance(token, numbers.Integral) or isinstance(token, bool):
-                    raise ValueError(f"token ids are integers, got {token!r}")
+                if type(token) is not int:       # (the common case needs no further look)
+                    if not isinstance(token, numbers.Integral) or isinstance(token, bool):
+                        raise ValueError(f"token ids are integers, got {token!r}")
+                    tokens[index] = token = int(token)
                 if not 0 <= token < vocab:
                     raise ValueError(f"token id {token!r} is outside the vocabulary of {vocab}")
-                tokens[index] = int(token)
             want = list(want)
             for w in want:
                 if not 0 <= w < len(tokens):
@@ -252,8 +253,7 @@ class Session:
         self._require_usable()
         seqs = self._validate(entries)
         growth = [(seq.slot, seq.start + seq.count) for seq in seqs]
-        self.cache.check_growth(growth)          # raises before anything changes
-        self.cache.grow(growth)
+        self.cache.grow(growth)                  # raises before anything changes
         saved = None
         try:
             captured = None
@@ -353,7 +353,7 @@ class Session:
         """The first step of a (bucket, bound) pair runs eagerly on the pair's own buffers and
         is then captured; later steps only refresh the metadata and replay."""
         seqs = ctx.sequences
-        layout = (captured.meta.layout(), captured.meta.capacity)
+        layout = captured.meta.generation
         if captured.graph is not None and captured.layout != layout:
             captured.graph = None           # the metadata moved: what was captured reads stale places
         if captured.graph is None:

@@ -10,6 +10,7 @@ still the same dot product.  Each projection may have a bias
 """
 from __future__ import annotations
 
+import functools
 import os
 
 import numpy as np
@@ -31,6 +32,18 @@ FUSED_DECODE = os.environ.get("EDGE_INFER_FUSED_DECODE", "1") != "0"
 TILE_US, MERGE_US, MERGE_SLICE_US = 1.9, 4.5, 0.1
 WAVE_SLOTS = 256 * 16         # waves the chip holds at once: compute units x waves a unit
 MAX_SLICES = 32
+
+
+@functools.lru_cache(maxsize=512)
+def _decode_items(n_seqs: int, live: int):
+    """One work item a sequence, [3, n_seqs]: sequence (-1: padding), its row, one position."""
+    seq = np.full(n_seqs, -1, dtype=np.int32)
+    seq[:live] = np.arange(live)
+    npos = np.zeros(n_seqs, dtype=np.int32)
+    npos[:live] = 1
+    items = np.stack([seq, np.arange(n_seqs, dtype=np.int32), npos])
+    items.setflags(write=False)
+    return items
 
 
 class Attention:
@@ -109,6 +122,11 @@ class Attention:
             return lib.attention_prefill_mfma_positions(self.group)
         return lib.attention_positions_per_item(self.group)
 
+    @property
+    def plan_key(self):
+        """Attention parts with equal keys plan the same sections."""
+        return ("attention", self.positions_per_item())
+
     def _items_section(self):
         return f"attention.items{self.positions_per_item()}"
 
@@ -118,12 +136,7 @@ class Attention:
         rows into items of `positions_per_item`, the ones with the longest key range first
         (they take longest, so they start first); a decode step has one item a sequence."""
         if plan.decode:
-            seq = np.full(plan.n_seqs, -1, dtype=np.int32)
-            seq[:plan.n_live_seqs] = np.arange(plan.n_live_seqs)
-            npos = np.zeros(plan.n_seqs, dtype=np.int32)
-            npos[:plan.n_live_seqs] = 1
-            items = np.stack([seq, np.arange(plan.n_seqs, dtype=np.int32), npos])
-            return {"attention.decode_items": items}
+            return {"attention.decode_items": _decode_items(plan.n_seqs, plan.n_live_seqs)}
         size = self.positions_per_item()
         items = []
         for index, seq in enumerate(plan.seqs):
