@@ -353,49 +353,65 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   }
 }
 
-// Prefill: a block of eight waves owns HB query heads of one kv group (HB = 4, 2 or 1, the
-// largest that divides the group) and 16 * (8 / HB) consecutive positions of one sequence;
-// a wave keeps 16 rows of one head as MFMA operands in registers (few enough registers for
-// two waves per SIMD, so that one wave's softmax runs beside the other's products) and
-// walks the key pages of the sequence.  A page of keys goes to LDS as stored, a page of
-// values goes to LDS transposed ([d][key]), once for the whole block, so the heads of a
-// group share every byte that is fetched.  Scores are computed transposed (S^T = K Q^T):
-// lane (c, n) then holds, for query row n, the keys 4c..4c+3 of every 16-key block, which is
-// exactly an A-operand register of P for the second product once two blocks are packed
-// together, so the probabilities never leave the registers.  Softmax state is float32 (in
-// units of log2); probabilities are rounded to bfloat16 for the value product (the
-// reference's prefill kernel does the same, operators/src/cuda/kernels/flash_attn_prefill.cu:240).
+// Prefill on 32x32x16 products.  A block of eight waves owns HB query heads of one kv group
+// (HB = 4, 2 or 1, the largest that divides the group) and 32 * (8 / HB) consecutive positions
+// of one sequence; a wave keeps 32 rows of one head as operands in registers and walks the key
+// pages of the sequence.  A page of keys and a page of values go to LDS once for the whole
+// block, so the heads of a group share every byte that is fetched; two pages alternate, so
+// that a page costs one barrier.  (A form with 16-row waves on 16x16x32 products, four waves
+// a SIMD, was measured against this one: an operand read from LDS feeds half the arithmetic
+// there and the instruction itself runs at a lower rate on this chip, 1.45 against 2.1
+// PFLOP/s in a loop of nothing else; it was 20 % slower from 3,000 tokens on and equal below.)
+//
+// S^T = K Q^T for a block of 32 keys: A = keys (lane (key l % 32, half l / 32) reads
+// k[key][16 s + 8 half .. +8] from LDS), B = the wave's queries in registers (lane (query
+// l % 32, half) holds q[query][16 s + 8 half .. +8]).  The result leaves lane (query n, half h)
+// with keys 8 i + 4 h + r of the block (i, r = 0..3): for a 16-key step t of the value
+// product these are keys 16 t + 4 h + r and 16 t + 8 + 4 h + r, eight values that are
+// exactly the lane's A operand of P, provided the values (B, lane (d column n, half h)) come
+// in the same order: two 8-byte reads of the transposed page at keys 16 t + 4 h and
+// 16 t + 8 + 4 h.  So the probabilities never leave the registers.  The two lanes of a query
+// share its running maximum (one exchange a page) and keep separate sums.  The output tile has
+// lane (d column n, half h) hold queries 8 i + 4 h + r, so factors per query (the rescaling
+// when a maximum moves, the final 1 / sum) pass through 32 floats of LDS a wave.  Softmax
+// state is float32 (in units of log2); probabilities are rounded to bfloat16 for the value
+// product (the reference's prefill kernel does the same,
+// operators/src/cuda/kernels/flash_attn_prefill.cu:240).
+//
+// Keys lie in LDS as stored, with the 16-byte chunks of a row exchanged among themselves
+// (chunk ^ key % 16, for 64-wide heads chunk ^ (key / 2) % 8) so that the 16 rows a quarter
+// of a wave reads touch every bank once; values lie transposed ([d][key]).
 // Blocks are numbered so that the blocks of one kv head fall on one XCD (the hardware deals
 // consecutive workgroups round-robin to its 8 XCDs): that head's keys and values then stay
 // in that XCD's L2.
-constexpr int kRowTiles = 1;     // 16-row tiles per wave
-constexpr int kPrefillWaves = 8; // two waves per SIMD: one's softmax overlaps the other's products
+constexpr int kPrefillWaves = 8;
 constexpr int kPrefillThreads = kPrefillWaves * EI_WAVE;
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+constexpr int kWideRows = 32;      // query rows of a wave
 
 template <int D, int HB>
-__global__ void __launch_bounds__(kPrefillThreads, 4)
+__global__ void __launch_bounds__(kPrefillThreads, 2)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
-                    const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
-                    const int32_t* __restrict__ item_row0, const int32_t* __restrict__ item_npos,
-                    int n_items, const int32_t* __restrict__ row_pos,
-                    const int32_t* __restrict__ page_table, int table_width,
-                    bf16_t* __restrict__ out, int nq, int nkv, int window, float scale,
-                    int pair) {
-  constexpr int DJ = D / 32;             // MFMA steps over d for the scores
-  constexpr int DB = D / 16;             // 16-wide output blocks over d
-  constexpr int KS = D + 8;              // LDS stride of a key row (elements)
+                         const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
+                         const int32_t* __restrict__ item_row0,
+                         const int32_t* __restrict__ item_npos, int n_items,
+                         const int32_t* __restrict__ row_pos,
+                         const int32_t* __restrict__ page_table, int table_width,
+                         bf16_t* __restrict__ out, int nq, int nkv, int window, float scale,
+                         int pair) {
+  constexpr int SJ = D / 16;             // 16-wide steps over d for the scores
+  constexpr int DB = D / 32;             // 32-wide output blocks over d
   constexpr int VS = EI_PAGE + 4;        // LDS stride of a transposed value row (34 dwords)
-  constexpr int CI = D / 64;             // 16-byte chunks per thread per page (D/8 * 64 / 512)
-  constexpr int RT = kRowTiles;
+  constexpr int CI = D / 64;             // 16-byte chunks per thread per page
+  constexpr int CHUNKS = D / 8;          // 16-byte chunks of a key row
+  constexpr int KBUF = EI_PAGE * D, VBUF = D * VS;    // elements of one page buffer
   // two pages of keys and of (transposed) values alternate, so that a page costs one barrier
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds2[2][EI_PAGE * KS];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds2[2][D * VS];
+  __shared__ __attribute__((aligned(16))) bf16_t k_lds[2 * KBUF];
+  __shared__ __attribute__((aligned(16))) bf16_t v_lds[2 * VBUF];
+  __shared__ __attribute__((aligned(16))) float factor_lds[kPrefillWaves][kWideRows];
 
-  // block number -> (kv head, head block, item) with the kv head fixed per XCD
   const int G = nq / nkv;
   const int head_blocks = G / HB;
-  // pair: a block takes item u and then item n - 1 - u, i.e. (the items being ordered by
-  // length) a long one and a short one, so that every block walks about as many pages
   const int units = pair ? (n_items + 1) / 2 : n_items;
   const int rests = units * head_blocks;
   int g, rest;
@@ -417,9 +433,31 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   if (rest >= rests) return;
   const int unit = rest / head_blocks, hb = rest % head_blocks;
   const int t = threadIdx.x, wave = t / EI_WAVE, lane = t % EI_WAVE;
-  const int r16 = lane & 15, c = lane >> 4;
+  const int n32 = lane & 31, half = lane >> 5;
   const int hw = wave % HB, pw = wave / HB;
   const int head = g * G + hb * HB + hw;
+  // a key row's chunk `chunk` lies at this place of the row
+  auto place = [](int key, int chunk) {
+    return CHUNKS == 16 ? (chunk ^ (key & 15)) : (chunk ^ ((key >> 1) & 7));
+  };
+  // Everything a lane needs to find its operands in a page buffer is worked out once: the
+  // places of its key chunks (they differ from step to step by the exchange of chunks; key
+  // blocks and buffers add constants), the place of its value words, and where its share of
+  // the next page goes.
+  int k_read[SJ];                        // (element offsets into the page buffers)
+#pragma unroll
+  for (int sj = 0; sj < SJ; ++sj) k_read[sj] = n32 * D + place(n32, 2 * sj + half) * 8;
+  const int v_read = n32 * VS + 4 * half;
+  const int ld_key = t >> 3, ld_dc = t & 7;
+  int k_write[CI], v_write[CI];
+#pragma unroll
+  for (int i = 0; i < CI; ++i) {
+    k_write[i] = ld_key * D + place(ld_key, ld_dc + 8 * i) * 8;
+    v_write[i] = ((ld_dc + 8 * i) * 8 + (ld_key & 1)) * VS + (ld_key & ~1);
+  }
+  const bool later = ld_dc & 4;
+  const uint32_t take = (ld_key & 1) ? 0x03020706u : 0x05040100u;   // bytes of (partner, own)
+
   for (int pass = 0; pass <= pair; ++pass) {
   const int item = pass == 0 ? unit : n_items - 1 - unit;
   if (pass == 1) {
@@ -430,227 +468,253 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   if (seq < 0) continue;
   const int row0 = item_row0[item], npos = item_npos[item];
 
-  // this lane's query rows (columns n of S^T), their positions, and the Q operands
-  int pos_r[RT];
-  bool row_valid[RT];
-  bf16x8 q_reg[RT][DJ];
+  // this lane's query (column n32 of S^T), its position, and the Q operand
+  const int my_row = pw * kWideRows + n32;
+  const bool row_valid = my_row < npos;
+  const int pos_q = row_valid ? row_pos[row0 + my_row] : -1;
+  bf16x8 q_reg[SJ];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const int my_row = pw * (16 * RT) + rt * 16 + r16;
-    row_valid[rt] = my_row < npos;
-    pos_r[rt] = row_valid[rt] ? row_pos[row0 + my_row] : -1;
-#pragma unroll
-    for (int j = 0; j < DJ; ++j) {
-      uint4 z = uint4{0u, 0u, 0u, 0u};
-      if (row_valid[rt])
-        z = *reinterpret_cast<const uint4*>(
-            q + (static_cast<size_t>(row0 + my_row) * nq + head) * D + j * 32 + c * 8);
-      q_reg[rt][j] = *reinterpret_cast<bf16x8*>(&z);
-    }
+  for (int sj = 0; sj < SJ; ++sj) {
+    uint4 z = uint4{0u, 0u, 0u, 0u};
+    if (row_valid)
+      z = *reinterpret_cast<const uint4*>(
+          q + (static_cast<size_t>(row0 + my_row) * nq + head) * D + sj * 16 + half * 8);
+    q_reg[sj] = *reinterpret_cast<bf16x8*>(&z);
   }
 
   const int first_pos = row_pos[row0], last_pos = row_pos[row0 + npos - 1];
   const int lo_key = window > 0 ? max(0, first_pos - window + 1) : 0;
   const int lo_page = lo_key / EI_PAGE, hi_page = last_pos / EI_PAGE;
-  // the rows of this wave: pw*32 .. pw*32+31 of the item
-  const bool wave_rows_valid = pw * (16 * RT) + 16 * RT <= npos;
-  const int wave_min_pos = wave_rows_valid ? row_pos[row0 + pw * (16 * RT)] : -1;
-  const int wave_max_pos = wave_rows_valid ? row_pos[row0 + pw * (16 * RT) + 16 * RT - 1] : -1;
+  const bool wave_rows_valid = pw * kWideRows + kWideRows <= npos;
+  const int wave_min_pos = wave_rows_valid ? row_pos[row0 + pw * kWideRows] : -1;
+  const int wave_max_pos = wave_rows_valid ? row_pos[row0 + pw * kWideRows + kWideRows - 1] : -1;
+  // a wave none of whose rows exist only helps to move pages
+  const bool wave_has_rows = pw * kWideRows < npos;
+  const int wave_last_pos = wave_has_rows
+      ? row_pos[row0 + min(npos, pw * kWideRows + kWideRows) - 1] : -1;
 
-  // scores are kept in units of log2 (scale * log2 e), so that 2^x is the exponential
   const float scale_log2 = scale * 1.4426950408889634f;
-  float m_run[RT], l_run[RT];
-  f32x4 o_acc[RT][DB];
+  float m_run = kLowest, l_run = 0.f;     // l_run: this lane's half of the keys only
+  f32x16 o_acc[DB];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    m_run[rt] = kLowest;
-    l_run[rt] = 0.f;
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int db = 0; db < DB; ++db) o_acc[rt][db] = f32x4{0.f, 0.f, 0.f, 0.f};
-  }
+    for (int e = 0; e < 16; ++e) o_acc[db][e] = 0.f;
 
-  // global -> register staging of a page: thread t takes key t/8, chunks (t%8) + 8*i
-  const int ld_key = t >> 3, ld_dc = t & 7;
   uint4 k_stage[CI], v_stage[CI];
-  // The physical page of the page after next is looked up while the next page's data is
-  // on its way, so that a page costs one trip to memory, not two in a row.
-  auto lookup = [&](int page_index) {
+  auto lookup = [&](int page_index) __attribute__((always_inline)) {
     return page_index <= hi_page
                ? page_table[static_cast<size_t>(seq) * table_width + page_index] : -1;
   };
-  auto load_page = [&](int page_index, int phys) {
+  auto load_page = [&](int page_index, int phys) __attribute__((always_inline)) {
     if (phys < 0) {                       // released by the window: every key is masked
 #pragma unroll
       for (int i = 0; i < CI; ++i) k_stage[i] = v_stage[i] = uint4{0u, 0u, 0u, 0u};
       return;
     }
-    const size_t base = ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D;
+    const size_t base = ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D + ld_dc * 8;
     const bool live = page_index * EI_PAGE + ld_key <= last_pos;   // later slots: stale bytes
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
-      const int dc = ld_dc + 8 * i;
-      k_stage[i] = live ? *reinterpret_cast<const uint4*>(k_pages + base + dc * 8)
+      k_stage[i] = live ? *reinterpret_cast<const uint4*>(k_pages + base + 64 * i)
                         : uint4{0u, 0u, 0u, 0u};
-      v_stage[i] = live ? *reinterpret_cast<const uint4*>(v_pages + base + dc * 8)
+      v_stage[i] = live ? *reinterpret_cast<const uint4*>(v_pages + base + 64 * i)
                         : uint4{0u, 0u, 0u, 0u};
     }
   };
-  auto store_page = [&](int buf) {
-    bf16_t* k_lds = k_lds2[buf];
-    bf16_t* v_lds = v_lds2[buf];
+  // Values go to LDS transposed ([d][key]).  A lane holds 8 values of one key as 4 dwords (d
+  // pairs); the lane 8 further in its row of 16 holds the same d of the next key, so after one
+  // exchange (a DPP rotation of the row by 8) the even-key lane owns the two keys of the even d
+  // of every pair and the odd-key lane those of the odd d: 4 dword stores a lane.  The upper 4
+  // lanes of a key take their d pairs one step later, which spreads the stores over the banks.
+  auto store_page = [&](auto buf_tag) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_tag)::value;
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
-      const int dc = ld_dc + 8 * i;
-      *reinterpret_cast<uint4*>(&k_lds[ld_key * KS + dc * 8]) = k_stage[i];
-      // Values go to LDS transposed ([d][key]).  A lane holds 8 values of one key as 4
-      // dwords (d pairs); the lane 8 further in its row of 16 holds the same d of the next
-      // key (keys come in even/odd pairs), so after one exchange (a DPP rotation of the row
-      // by 8) the even-key lane owns the two keys of the even d of every pair and the odd-key
-      // lane those of the odd d: 4 dword stores a lane instead of 8 halfword stores.  The 8
-      // lanes of a key write rows 8 apart, which a row stride of 34 dwords would put on 4
-      // banks; the upper 4 lanes take their d pairs one step later, which doubles that.
+      *reinterpret_cast<uint4*>(&k_lds[k_write[i] + buf * KBUF]) = k_stage[i];
       const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
-      uint32_t pw[4];
+      uint32_t partner[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        pw[e] = __builtin_amdgcn_update_dpp(0u, w[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
-      const bool odd_key = ld_key & 1;
-      const bool later = ld_dc & 4;
-      const uint32_t take = odd_key ? 0x03020706u : 0x05040100u;   // bytes of (partner, own)
-      const int column = ld_key & ~1;
+        partner[e] = __builtin_amdgcn_update_dpp(0u, w[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
+      uint32_t both[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) both[e] = __builtin_amdgcn_perm(partner[e], w[e], take);
+      // d pair e goes to row 2 e (+ the odd key's 1) of the chunk; the later lanes start at pair 1
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int e2 = (e + 1) & 3;
-        const uint32_t own = later ? w[e2] : w[e];
-        const uint32_t other = later ? pw[e2] : pw[e];
-        const int pair_index = later ? e2 : e;
-        // even key: (own.lo, partner.lo) = d even of keys (k, k+1); odd key: (partner.hi, own.hi)
-        const uint32_t both = __builtin_amdgcn_perm(other, own, take);
-        const int d = dc * 8 + 2 * pair_index + (odd_key ? 1 : 0);
-        *reinterpret_cast<uint32_t*>(&v_lds[d * VS + column]) = both;
+        const uint32_t word = later ? both[e2] : both[e];
+        const int to = v_write[i] + buf * VBUF + (later ? 2 * e2 * VS : 2 * e * VS);
+        *reinterpret_cast<uint32_t*>(&v_lds[to]) = word;
       }
     }
   };
 
-  // Page p is multiplied from LDS buffer p & 1 while page p + 1 (fetched a page ago) goes
-  // from registers into the other buffer and page p + 2 is requested; the barrier at the
-  // end of a page says both that the other buffer is complete and that this one is free.
-  load_page(lo_page, lookup(lo_page));
-  store_page(lo_page & 1);
-  load_page(lo_page + 1, lookup(lo_page + 1));    // zeros past the last page
-  int phys_next = lookup(lo_page + 2);
-  __syncthreads();
-  for (int page = lo_page; page <= hi_page; ++page) {
-    const bf16_t* k_lds = k_lds2[page & 1];
-    const bf16_t* v_lds = v_lds2[page & 1];
-    const int key_base = page * EI_PAGE;
-
-    // pages that every row of this wave sees in full (all but the last one or two of a
-    // causal prompt) need no mask
-    const bool no_mask = wave_rows_valid && key_base + EI_PAGE - 1 <= wave_min_pos &&
-                         (window <= 0 || key_base > wave_max_pos - window);
-    bf16x8 p_reg[RT][2];                  // A operands of P for the two 32-key steps
-    // One row tile after the other, to keep few registers alive: scores, softmax, and
-    // (only if its maximum moved) the rescaling of that tile's output.
+  // The scores of one page from LDS buffer `buf`, their softmax into `p_reg` (A operands of P
+  // for the four 16-key steps), and the rescaling of the output so far.  MASKED: some key of
+  // the page is hidden from some row of the wave (all but the last one or two pages of a
+  // causal prompt need no mask).
+  bf16x8 p_reg[4];
+  auto scores = [&](const int key_base, auto buf_tag, const bool MASKED) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_tag)::value;
+    f32x16 s[2];
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt) {
-      // S^T blocks: lane (c, n) holds keys key_base + kb*16 + 4c + r for query row n
-      f32x4 s[4];
+    for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
-      for (int kb = 0; kb < 4; ++kb) {
-        s[kb] = f32x4{0.f, 0.f, 0.f, 0.f};
+      for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
 #pragma unroll
-        for (int j = 0; j < DJ; ++j) {
-          const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
-              &k_lds[(kb * 16 + r16) * KS + j * 32 + c * 8]);
-          s[kb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, q_reg[rt][j], s[kb], 0, 0, 0);
+      for (int sj = 0; sj < SJ; ++sj) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&k_lds[k_read[sj] + buf * KBUF + kb * 32 * D]);
+        s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q_reg[sj], s[kb], 0, 0, 0);
+      }
+    }
+    if (MASKED) {
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int key = key_base + kb * 32 + 8 * i + 4 * half + r;
+            const bool visible = key <= pos_q && (window <= 0 || key > pos_q - window);
+            if (!visible) s[kb][4 * i + r] = -INFINITY;     // (pos_q = -1: a row that is not there)
+          }
+    }
+    float tile_max = fmaxf(s[0][0], s[1][0]);
+#pragma unroll
+    for (int e = 1; e < 16; ++e) tile_max = fmaxf(tile_max, fmaxf(s[0][e], s[1][e]));
+    {   // the other half of this query's keys sits 32 lanes away
+      ei::ei_u32x2 both = __builtin_amdgcn_permlane32_swap(__float_as_uint(tile_max),
+                                                           __float_as_uint(tile_max), false, false);
+      tile_max = fmaxf(__uint_as_float(both.x), __uint_as_float(both.y));
+    }
+    // running maximum in units of log2 (raw score * scale * log2 e; the scale is positive);
+    // a row with no visible key yet keeps the lowest value, not -inf, so that no NaN arises
+    const float m_new = fmaxf(m_run, tile_max * scale_log2);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    float tile_sum = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+      for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int e = 4 * (2 * tt + (j >> 2)) + (j & 3);
+          const float p = __builtin_amdgcn_exp2f(fmaf(s[kb][e], scale_log2, -m_new));
+          tile_sum += p;
+          p_reg[2 * kb + tt][j] = static_cast<__bf16>(p);
+        }
+    l_run = l_run * alpha + tile_sum;
+    m_run = m_new;
+    if (__any(alpha != 1.f)) {            // the maximum of some row of this wave has moved
+      if (half == 0) factor_lds[wave][n32] = alpha;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float4 a = *reinterpret_cast<const float4*>(&factor_lds[wave][8 * i + 4 * half]);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          o_acc[db][4 * i + 0] *= a.x;
+          o_acc[db][4 * i + 1] *= a.y;
+          o_acc[db][4 * i + 2] *= a.z;
+          o_acc[db][4 * i + 3] *= a.w;
         }
       }
-      if (!no_mask) {
-#pragma unroll
-        for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int key = key_base + kb * 16 + 4 * c + r;
-            const bool visible = row_valid[rt] && key <= pos_r[rt] &&
-                                 (window <= 0 || key > pos_r[rt] - window);
-            if (!visible) s[kb][r] = -INFINITY;
-          }
-      }
-      float tile_max = -INFINITY;
-#pragma unroll
-      for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) tile_max = fmaxf(tile_max, s[kb][r]);
-      tile_max = ei::rows_max(tile_max);
-      // running maximum in units of log2 (raw score * scale * log2 e; the scale is positive)
-      const float m_new = fmaxf(m_run[rt], tile_max * scale_log2);
-      const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
-      float tile_sum = 0.f;
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-        for (int half = 0; half < 2; ++half)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const float p = __builtin_amdgcn_exp2f(fmaf(s[2 * ks + half][r], scale_log2, -m_new));
-            tile_sum += p;
-            p_reg[rt][ks][half * 4 + r] = static_cast<__bf16>(p);
-          }
-      }
-      tile_sum = ei::rows_sum(tile_sum);
-      l_run[rt] = l_run[rt] * alpha + tile_sum;
-      m_run[rt] = m_new;
-      if (__any(alpha != 1.f)) {            // the maximum of some row of this tile has moved
-        // the output rows of this lane are query rows 4c + r: fetch their factors
-        float a_row[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) a_row[r] = __shfl(alpha, 4 * c + r, EI_WAVE);
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-          for (int r = 0; r < 4; ++r) o_acc[rt][db][r] *= a_row[r];
-      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
+  };
+  // output += P V for the page whose probabilities are in `p_reg`, values from buffer `buf`
+  auto values = [&](auto buf_tag) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_tag)::value;
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int st = 0; st < 4; ++st) {
 #pragma unroll
-      for (int ks = 0; ks < 2; ++ks) {
-        // values: lane (n = d column, c) supplies keys ks*32 + {4c..4c+3} and +16
-        const bf16_t* vrow = &v_lds[(db * 16 + r16) * VS + ks * 32 + 4 * c];
+      for (int db = 0; db < DB; ++db) {
+        const bf16_t* vrow = &v_lds[v_read + buf * VBUF + db * 32 * VS + st * 16];
         const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 16);
+        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
         uint4 both = uint4{lo.x, lo.y, hi.x, hi.y};
         const bf16x8 vf = *reinterpret_cast<bf16x8*>(&both);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-          o_acc[rt][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(p_reg[rt][ks], vf,
-                                                                  o_acc[rt][db], 0, 0, 0);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p_reg[st], vf, o_acc[db], 0, 0, 0);
       }
     }
+  };
+  // whether this wave has anything to do with a page: one that lies wholly after the wave's
+  // last row (the item's later rows need it) or wholly before its window is only moved
+  auto page_seen = [&](const int page) __attribute__((always_inline)) {
+    const int key_base = page * EI_PAGE;
+    return wave_has_rows && key_base <= wave_last_pos &&
+           (window <= 0 || !wave_rows_valid || key_base + EI_PAGE - 1 > wave_min_pos - window);
+  };
+  auto scores_of = [&](const int page, auto buf_tag) __attribute__((always_inline)) {
+    const int key_base = page * EI_PAGE;
+    const bool no_mask = wave_rows_valid && key_base + EI_PAGE - 1 <= wave_min_pos &&
+                         (window <= 0 || key_base > wave_max_pos - window);
+    scores(key_base, buf_tag, !no_mask);
+  };
+  // Page p is multiplied from buffer p & 1 while page p + 1 (fetched a page ago) goes from
+  // registers into the other buffer and page p + 2 is requested; the barrier at the end of a
+  // page says both that the other buffer is complete and that this one is free.
+  int phys_next;
+  auto one_page = [&](const int page, auto buf_tag) __attribute__((always_inline)) {
+    constexpr int buf = decltype(buf_tag)::value;
+    if (page_seen(page)) {
+      scores_of(page, buf_tag);
+      values(buf_tag);
+    }
     if (page < hi_page) {
-      store_page((page + 1) & 1);
+      store_page(std::integral_constant<int, 1 - buf>{});
       load_page(page + 2, phys_next);
       phys_next = lookup(page + 3);
       __syncthreads();
     }
+  };
+  load_page(lo_page, lookup(lo_page));
+  if (lo_page & 1) store_page(std::integral_constant<int, 1>{});
+  else store_page(std::integral_constant<int, 0>{});
+  load_page(lo_page + 1, lookup(lo_page + 1));    // zeros past the last page
+  phys_next = lookup(lo_page + 2);
+  __syncthreads();
+  int page = lo_page;
+  if (page & 1) {
+    one_page(page, std::integral_constant<int, 1>{});
+    ++page;
+  }
+  for (; page <= hi_page; page += 2) {
+    one_page(page, std::integral_constant<int, 0>{});
+    if (page + 1 <= hi_page) one_page(page + 1, std::integral_constant<int, 1>{});
   }
 
-  // lane (c, n) holds O[query row 4c + r][d = db*16 + n]
+  // 1 / sum per query through LDS; lane (d column n32, half) holds O[query 8 i + 4 half + r]
+  {
+    ei::ei_u32x2 both = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run),
+                                                         __float_as_uint(l_run), false, false);
+    const float l = __uint_as_float(both.x) + __uint_as_float(both.y);
+    if (half == 0) factor_lds[wave][n32] = l > 0.f ? 1.f / l : 0.f;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  }
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
+  for (int i = 0; i < 4; ++i) {
+    const float4 inv4 = *reinterpret_cast<const float4*>(&factor_lds[wave][8 * i + 4 * half]);
+    const float inv[4] = {inv4.x, inv4.y, inv4.z, inv4.w};
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      const float l = __shfl(l_run[rt], 4 * c + r, EI_WAVE);
-      const float inv = l > 0.f ? 1.f / l : 0.f;
-      const int orow = pw * (16 * RT) + rt * 16 + 4 * c + r;
+      const int orow = pw * kWideRows + 8 * i + 4 * half + r;
       if (orow >= npos) continue;
       bf16_t* dst = out + (static_cast<size_t>(row0 + orow) * nq + head) * D;
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        dst[db * 16 + r16] = ei::from_f32<bf16_t>(o_acc[rt][db][r] * inv);
+        dst[db * 32 + n32] = ei::from_f32<bf16_t>(o_acc[db][4 * i + r] * inv[r]);
     }
   }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
   }  // pass
 }
 
@@ -723,15 +787,16 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
 // Positions of one sequence that a prefill work item of this file holds for a group ratio.
 extern "C" int ei_attn_prefill_mfma_positions(int G) {
   const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
-  return 16 * kRowTiles * (kPrefillWaves / HB);
+  return kWideRows * (kPrefillWaves / HB);
 }
 
 template <int D, int HB>
 static void launch_prefill(int blocks, hipStream_t stream, const bf16_t* q, const bf16_t* k,
-                           const bf16_t* v, const int32_t* item_seq, const int32_t* item_row0,
-                           const int32_t* item_npos, int n_items, const int32_t* row_pos,
-                           const int32_t* page_table, int table_width, bf16_t* out, int nq,
-                           int nkv, int window, float scale, int pair) {
+                                const bf16_t* v, const int32_t* item_seq,
+                                const int32_t* item_row0, const int32_t* item_npos, int n_items,
+                                const int32_t* row_pos, const int32_t* page_table,
+                                int table_width, bf16_t* out, int nq, int nkv, int window,
+                                float scale, int pair) {
   attn_prefill_kernel<D, HB><<<blocks, kPrefillThreads, 0, stream>>>(
       q, k, v, item_seq, item_row0, item_npos, n_items, row_pos, page_table, table_width, out,
       nq, nkv, window, scale, pair);

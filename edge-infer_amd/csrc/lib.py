@@ -313,16 +313,17 @@ def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
 
 
 def attention_prefill_mfma_positions(group: int) -> int:
-    """Positions of a sequence per work item of the matrix-core prefill kernel: a block
-    holds 4, 2 or 1 heads of a kv group and 32 positions for each of its 4 waves."""
+    """Positions of a sequence per work item of the matrix-core prefill kernel: a block of 8
+    waves holds 4, 2 or 1 heads of a kv group, each wave 32 positions of one head."""
     heads = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
-    return 32 * (4 // heads)
+    return 32 * (8 // heads)
 
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                            page_table, out, n_heads, n_kv_heads, head_dim, window=None,
                            scale=None) -> None:
-    """bfloat16 prefill attention on the matrix cores; items hold up to 64 positions."""
+    """bfloat16 prefill attention on the matrix cores; an item holds up to
+    `attention_prefill_mfma_positions(group)` positions of one sequence."""
     lib = library("attention_mfma")
     n = q.shape[0]
     if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
