@@ -358,7 +358,13 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
 // of one sequence; a wave keeps 32 rows of one head as operands in registers and walks the key
 // pages of the sequence.  A page of keys and a page of values go to LDS once for the whole
 // block, so the heads of a group share every byte that is fetched; two pages alternate, so
-// that a page costs one barrier.  (A form with 16-row waves on 16x16x32 products, four waves
+// that a page costs one barrier.  KW = 2: the eight waves are HB heads x half as many groups of
+// rows x 2 halves of every page's keys; the wave of the second half hands its maximum, sum and
+// output tile to the wave of the first through LDS at the end.  Work items are then half as
+// long, so a short prompt gives twice the blocks, enough for the pairing of a long item with a
+// short one below (one 2,048-token prompt of 32/8 heads: 72 against 82 us).  With enough blocks
+// without it KW = 1 is faster (what a page costs a wave beside its products is not halved).
+// (A form with 16-row waves on 16x16x32 products, four waves
 // a SIMD, was measured against this one: an operand read from LDS feeds half the arithmetic
 // there and the instruction itself runs at a lower rate on this chip, 1.45 against 2.1
 // PFLOP/s in a loop of nothing else; it was 20 % slower from 3,000 tokens on and equal below.)
@@ -388,8 +394,9 @@ constexpr int kPrefillWaves = 8;
 constexpr int kPrefillThreads = kPrefillWaves * EI_WAVE;
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 constexpr int kWideRows = 32;      // query rows of a wave
+constexpr int kAhead = 3;          // LDS operand reads in flight before the product that needs the first
 
-template <int D, int HB>
+template <int D, int HB, int KW>
 __global__ void __launch_bounds__(kPrefillThreads, 2)
 attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                          const bf16_t* __restrict__ v_pages, const int32_t* __restrict__ item_seq,
@@ -405,10 +412,22 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   constexpr int CI = D / 64;             // 16-byte chunks per thread per page
   constexpr int CHUNKS = D / 8;          // 16-byte chunks of a key row
   constexpr int KBUF = EI_PAGE * D, VBUF = D * VS;    // elements of one page buffer
+  constexpr int NG = kPrefillWaves / (HB * KW);       // groups of 32 rows in a block
+  constexpr int KBL = 2 / KW;            // blocks of 32 keys of a page that a wave takes
+  static_assert(KW == 1 || KW == 2, "a page's keys go to one wave or to two");
+  static_assert(NG >= 1, "eight waves: heads x row groups x key ways");
   // two pages of keys and of (transposed) values alternate, so that a page costs one barrier
-  __shared__ __attribute__((aligned(16))) bf16_t k_lds[2 * KBUF];
-  __shared__ __attribute__((aligned(16))) bf16_t v_lds[2 * VBUF];
+  __shared__ __attribute__((aligned(16))) bf16_t page_lds[2 * KBUF + 2 * VBUF];
+  bf16_t* const k_lds = page_lds;
+  bf16_t* const v_lds = page_lds + 2 * KBUF;
   __shared__ __attribute__((aligned(16))) float factor_lds[kPrefillWaves][kWideRows];
+  // (KW = 2) what the second wave of a (head, rows) pair hands to the first at the end: its
+  // running maximum and sum per row here, its output tile in the page buffers
+  __shared__ float handed_lds[KW == 2 ? kPrefillWaves / 2 : 1][2][kWideRows];
+  __shared__ __attribute__((aligned(16))) float other_lds[KW == 2 ? kPrefillWaves : 1][kWideRows];
+  static_assert(KW == 1 || (kPrefillWaves / 2) * (D / 32) * 16 * EI_WAVE * sizeof(float) <=
+                               sizeof(bf16_t) * (2 * KBUF + 2 * VBUF),
+                "the handed-over output tiles fit the page buffers");
 
   const int G = nq / nkv;
   const int head_blocks = G / HB;
@@ -434,7 +453,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   const int unit = rest / head_blocks, hb = rest % head_blocks;
   const int t = threadIdx.x, wave = t / EI_WAVE, lane = t % EI_WAVE;
   const int n32 = lane & 31, half = lane >> 5;
-  const int hw = wave % HB, pw = wave / HB;
+  const int hw = wave % HB, pw = (wave / HB) % NG, kw = wave / (HB * NG);
   const int head = g * G + hb * HB + hw;
   // a key row's chunk `chunk` lies at this place of the row
   auto place = [](int key, int chunk) {
@@ -555,35 +574,50 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   // for the four 16-key steps), and the rescaling of the output so far.  MASKED: some key of
   // the page is hidden from some row of the wave (all but the last one or two pages of a
   // causal prompt need no mask).
-  bf16x8 p_reg[4];
+  bf16x8 p_reg[2 * KBL];
   auto scores = [&](const int key_base, auto buf_tag, const bool MASKED) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
-    f32x16 s[2];
+    f32x16 s[KBL];
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb) {
+    for (int kb = 0; kb < KBL; ++kb)
 #pragma unroll
       for (int e = 0; e < 16; ++e) s[kb][e] = 0.f;
 #pragma unroll
-      for (int sj = 0; sj < SJ; ++sj) {
-        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(&k_lds[k_read[sj] + buf * KBUF + kb * 32 * D]);
+    for (int sj = 0; sj < SJ; ++sj)
+#pragma unroll
+      for (int kb = 0; kb < KBL; ++kb) {
+        const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
+            &k_lds[k_read[sj] + buf * KBUF + (kw * KBL + kb) * 32 * D]);
         s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q_reg[sj], s[kb], 0, 0, 0);
       }
+    // instruction order: the operand reads from LDS run kAhead products ahead of the products
+    // that take them (0x100: LDS reads, 0x008: matrix products)
+    __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);
+#pragma unroll
+    for (int n = 0; n < SJ * KBL; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
     }
     if (MASKED) {
+      // (an empty statement the compiler may not move: it keeps this a branch, which all but
+      // the last pages of a causal prompt jump over, instead of 128 predicated instructions)
+      asm volatile("");
 #pragma unroll
-      for (int kb = 0; kb < 2; ++kb)
+      for (int kb = 0; kb < KBL; ++kb)
 #pragma unroll
         for (int i = 0; i < 4; ++i)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
-            const int key = key_base + kb * 32 + 8 * i + 4 * half + r;
+            const int key = key_base + (kw * KBL + kb) * 32 + 8 * i + 4 * half + r;
             const bool visible = key <= pos_q && (window <= 0 || key > pos_q - window);
             if (!visible) s[kb][4 * i + r] = -INFINITY;     // (pos_q = -1: a row that is not there)
           }
     }
-    float tile_max = fmaxf(s[0][0], s[1][0]);
+    float tile_max = s[0][0];
 #pragma unroll
-    for (int e = 1; e < 16; ++e) tile_max = fmaxf(tile_max, fmaxf(s[0][e], s[1][e]));
+    for (int kb = 0; kb < KBL; ++kb)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) tile_max = fmaxf(tile_max, s[kb][e]);
     {   // the other half of this query's keys sits 32 lanes away
       ei::ei_u32x2 both = __builtin_amdgcn_permlane32_swap(__float_as_uint(tile_max),
                                                            __float_as_uint(tile_max), false, false);
@@ -595,7 +629,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float tile_sum = 0.f;
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < KBL; ++kb)
 #pragma unroll
       for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
@@ -631,10 +665,10 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   auto values = [&](auto buf_tag) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
 #pragma unroll
-    for (int st = 0; st < 4; ++st) {
+    for (int st = 0; st < 2 * KBL; ++st) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const bf16_t* vrow = &v_lds[v_read + buf * VBUF + db * 32 * VS + st * 16];
+        const bf16_t* vrow = &v_lds[v_read + buf * VBUF + db * 32 * VS + (kw * 2 * KBL + st) * 16];
         const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
         const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
         uint4 both = uint4{lo.x, lo.y, hi.x, hi.y};
@@ -642,18 +676,26 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
         o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p_reg[st], vf, o_acc[db], 0, 0, 0);
       }
     }
+    __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);      // as for the scores
+#pragma unroll
+    for (int n = 0; n < 2 * KBL * DB; ++n) {
+      __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+    }
   };
   // whether this wave has anything to do with a page: one that lies wholly after the wave's
   // last row (the item's later rows need it) or wholly before its window is only moved
+  // (the wave's keys of a page: KBL blocks of 32 from block kw * KBL on)
   auto page_seen = [&](const int page) __attribute__((always_inline)) {
-    const int key_base = page * EI_PAGE;
-    return wave_has_rows && key_base <= wave_last_pos &&
-           (window <= 0 || !wave_rows_valid || key_base + EI_PAGE - 1 > wave_min_pos - window);
+    const int key_lo = page * EI_PAGE + kw * KBL * 32, key_hi = key_lo + KBL * 32 - 1;
+    return wave_has_rows && key_lo <= wave_last_pos &&
+           (window <= 0 || !wave_rows_valid || key_hi > wave_min_pos - window);
   };
   auto scores_of = [&](const int page, auto buf_tag) __attribute__((always_inline)) {
     const int key_base = page * EI_PAGE;
-    const bool no_mask = wave_rows_valid && key_base + EI_PAGE - 1 <= wave_min_pos &&
-                         (window <= 0 || key_base > wave_max_pos - window);
+    const int key_lo = key_base + kw * KBL * 32, key_hi = key_lo + KBL * 32 - 1;
+    const bool no_mask = wave_rows_valid && key_hi <= wave_min_pos &&
+                         (window <= 0 || key_lo > wave_max_pos - window);
     scores(key_base, buf_tag, !no_mask);
   };
   // Page p is multiplied from buffer p & 1 while page p + 1 (fetched a page ago) goes from
@@ -690,27 +732,76 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   }
 
   // 1 / sum per query through LDS; lane (d column n32, half) holds O[query 8 i + 4 half + r]
+  float l_wave;
   {
     ei::ei_u32x2 both = __builtin_amdgcn_permlane32_swap(__float_as_uint(l_run),
                                                          __float_as_uint(l_run), false, false);
-    const float l = __uint_as_float(both.x) + __uint_as_float(both.y);
-    if (half == 0) factor_lds[wave][n32] = l > 0.f ? 1.f / l : 0.f;
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    l_wave = __uint_as_float(both.x) + __uint_as_float(both.y);
   }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const float4 inv4 = *reinterpret_cast<const float4*>(&factor_lds[wave][8 * i + 4 * half]);
-    const float inv[4] = {inv4.x, inv4.y, inv4.z, inv4.w};
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int orow = pw * kWideRows + 8 * i + 4 * half + r;
-      if (orow >= npos) continue;
-      bf16_t* dst = out + (static_cast<size_t>(row0 + orow) * nq + head) * D;
+  float own_factor = l_wave > 0.f ? 1.f / l_wave : 0.f;   // what this wave's output is scaled by
+  float other_factor = 0.f;                               // and the handed-over one
+  if constexpr (KW == 2) {
+    // The wave of the second half of every page's keys hands its state to the wave of the
+    // first: o = (o_0 2^(m_0 - m) + o_1 2^(m_1 - m)) / (l_0 2^(m_0 - m) + l_1 2^(m_1 - m)).
+    float* const tile_lds = reinterpret_cast<float*>(page_lds);
+    const int couple = wave % (HB * NG);
+    __syncthreads();                       // every wave has read the last page
+    if (kw == 1) {
 #pragma unroll
       for (int db = 0; db < DB; ++db)
-        dst[db * 32 + n32] = ei::from_f32<bf16_t>(o_acc[db][4 * i + r] * inv[r]);
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          tile_lds[((couple * DB + db) * 16 + e) * EI_WAVE + lane] = o_acc[db][e];
+      if (half == 0) {
+        handed_lds[couple][0][n32] = m_run;
+        handed_lds[couple][1][n32] = l_wave;
+      }
+    }
+    __syncthreads();
+    if (kw == 0) {
+      const float m_other = handed_lds[couple][0][n32], l_other = handed_lds[couple][1][n32];
+      const float m = fmaxf(m_run, m_other);
+      const float f_own = __builtin_amdgcn_exp2f(m_run - m);
+      const float f_other = __builtin_amdgcn_exp2f(m_other - m);
+      const float l = l_wave * f_own + l_other * f_other;
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      own_factor = f_own * inv;
+      other_factor = f_other * inv;
+    }
+  }
+  if (half == 0) {
+    factor_lds[wave][n32] = own_factor;
+    if constexpr (KW == 2) other_lds[wave][n32] = other_factor;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (kw == 0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float4 inv4 = *reinterpret_cast<const float4*>(&factor_lds[wave][8 * i + 4 * half]);
+      const float inv[4] = {inv4.x, inv4.y, inv4.z, inv4.w};
+      float add[4] = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (KW == 2) {
+        const float4 add4 = *reinterpret_cast<const float4*>(&other_lds[wave][8 * i + 4 * half]);
+        add[0] = add4.x; add[1] = add4.y; add[2] = add4.z; add[3] = add4.w;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int orow = pw * kWideRows + 8 * i + 4 * half + r;
+        if (orow >= npos) continue;
+        bf16_t* dst = out + (static_cast<size_t>(row0 + orow) * nq + head) * D;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          float o = o_acc[db][4 * i + r] * inv[r];
+          if constexpr (KW == 2) {
+            const float* const tile_lds = reinterpret_cast<const float*>(page_lds);
+            o = fmaf(tile_lds[(((wave % (HB * NG)) * DB + db) * 16 + 4 * i + r) * EI_WAVE + lane],
+                     add[r], o);
+          }
+          dst[db * 32 + n32] = ei::from_f32<bf16_t>(o);
+        }
+      }
     }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -784,32 +875,37 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
 
 }  // namespace
 
-// Positions of one sequence that a prefill work item of this file holds for a group ratio.
+// Positions of one sequence that a prefill work item of this file holds for a group ratio
+// (with key_ways = 2, half as many: two waves then share the keys of every page for the same
+// rows, which gives a short prompt twice the blocks).
 extern "C" int ei_attn_prefill_mfma_positions(int G) {
   const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
   return kWideRows * (kPrefillWaves / HB);
 }
 
-template <int D, int HB>
+template <int D, int HB, int KW>
 static void launch_prefill(int blocks, hipStream_t stream, const bf16_t* q, const bf16_t* k,
                                 const bf16_t* v, const int32_t* item_seq,
                                 const int32_t* item_row0, const int32_t* item_npos, int n_items,
                                 const int32_t* row_pos, const int32_t* page_table,
                                 int table_width, bf16_t* out, int nq, int nkv, int window,
                                 float scale, int pair) {
-  attn_prefill_kernel<D, HB><<<blocks, kPrefillThreads, 0, stream>>>(
+  attn_prefill_kernel<D, HB, KW><<<blocks, kPrefillThreads, 0, stream>>>(
       q, k, v, item_seq, item_row0, item_npos, n_items, row_pos, page_table, table_width, out,
       nq, nkv, window, scale, pair);
 }
 
 // q, out: [N, nq, D] bfloat16; items: (sequence, first packed row, positions), each holding
-// at most ei_attn_prefill_mfma_positions(nq / nkv) positions.
+// at most ei_attn_prefill_mfma_positions(nq / nkv) / key_ways positions (key_ways 1 or 2; the
+// kernel does not see an item's size, so items that are too large would lose rows: the
+// caller, who makes them, is bound to it).
 extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, const void* v_pages,
                                          const int32_t* item_seq, const int32_t* item_row0,
                                          const int32_t* item_npos, int n_items,
                                          const int32_t* row_pos, const int32_t* page_table,
                                          int table_width, void* out, int nq, int nkv, int D,
-                                         int window, float scale, hipStream_t stream) {
+                                         int window, float scale, int key_ways,
+                                         hipStream_t stream) {
   EI_REQUIRE(n_items > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_prefill: bad sizes");
   EI_REQUIRE(D == 64 || D == 128, "attention_prefill: this kernel takes head_dim 64 or 128");
   EI_REQUIRE(q && k_pages && v_pages && item_seq && item_row0 && item_npos && row_pos &&
@@ -818,6 +914,8 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
   EI_REQUIRE(window >= 0, "attention_prefill: negative window");
   const int G = nq / nkv;
   const int HB = G % 4 == 0 ? 4 : (G % 2 == 0 ? 2 : 1);
+  EI_REQUIRE(key_ways == 1 || (key_ways == 2 && HB * 2 <= kPrefillWaves),
+             "attention_prefill: key_ways must be 1 or 2");
   // Enough blocks to fill the chip twice over: pair a long item with a short one per block
   // (the caller orders the items by length, longest first), so that the blocks take about
   // equally long; with fewer blocks the pairs would leave compute units empty.
@@ -834,9 +932,16 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
   const bf16_t* vv = static_cast<const bf16_t*>(v_pages);
   bf16_t* oo = static_cast<bf16_t*>(out);
 #define EI_PREFILL(DD, HH)                                                                    \
-  launch_prefill<DD, HH>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq, item_row0,   \
-                         item_npos, n_items, row_pos, page_table, table_width, oo, nq, nkv,   \
-                         window, scale, pair)
+  do {                                                                                        \
+    if (key_ways == 2)                                                                        \
+      launch_prefill<DD, HH, 2>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq,       \
+                                item_row0, item_npos, n_items, row_pos, page_table,           \
+                                table_width, oo, nq, nkv, window, scale, pair);               \
+    else                                                                                      \
+      launch_prefill<DD, HH, 1>(static_cast<int>(blocks), stream, qq, kk, vv, item_seq,       \
+                                item_row0, item_npos, n_items, row_pos, page_table,           \
+                                table_width, oo, nq, nkv, window, scale, pair);               \
+  } while (0)
   if (D == 64) {
     if (HB == 4) EI_PREFILL(64, 4); else if (HB == 2) EI_PREFILL(64, 2); else EI_PREFILL(64, 1);
   } else {

@@ -49,7 +49,7 @@ _SIGNATURES = {
         "ei_attn_prefill_mfma_positions": [c_int],
         "ei_attention_prefill_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-                                      c_int, c_int, c_float, c_void_p],
+                                      c_int, c_int, c_float, c_int, c_void_p],
         "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
@@ -312,18 +312,22 @@ def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
     return head_dim in MFMA_HEAD_DIMS and group >= 1
 
 
-def attention_prefill_mfma_positions(group: int) -> int:
+def attention_prefill_mfma_positions(group: int, key_ways: int = 1) -> int:
     """Positions of a sequence per work item of the matrix-core prefill kernel: a block of 8
-    waves holds 4, 2 or 1 heads of a kv group, each wave 32 positions of one head."""
+    waves holds 4, 2 or 1 heads of a kv group, each wave 32 positions of one head; with
+    `key_ways` = 2 two waves share the keys of every page for the same positions, so an item
+    is half as long (0: the group has no such form)."""
     heads = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
-    return 32 * (8 // heads)
+    if key_ways not in (1, 2) or heads * key_ways > 8:
+        return 0
+    return 32 * (8 // (heads * key_ways))
 
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                            page_table, out, n_heads, n_kv_heads, head_dim, window=None,
-                           scale=None) -> None:
+                           scale=None, key_ways=1) -> None:
     """bfloat16 prefill attention on the matrix cores; an item holds up to
-    `attention_prefill_mfma_positions(group)` positions of one sequence."""
+    `attention_prefill_mfma_positions(group, key_ways)` positions of one sequence."""
     lib = library("attention_mfma")
     n = q.shape[0]
     if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
@@ -342,7 +346,7 @@ def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, 
         n_items, _gpu(row_pos, "row_pos", torch.int32),
         _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
         _gpu(out, "out", torch.bfloat16), n_heads, n_kv_heads, head_dim, int(window or 0),
-        float(scale), _stream())
+        float(scale), int(key_ways), _stream())
     _check(lib, status, "attention_prefill")
 
 

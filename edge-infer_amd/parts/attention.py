@@ -117,18 +117,33 @@ class Attention:
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
 
     # the number of positions of one sequence that a prefill work item covers
-    def positions_per_item(self):
+    def positions_per_item(self, key_ways: int = 1):
         if self.matrix_cores:          # the matrix-core prefill kernel takes the same cases
-            return lib.attention_prefill_mfma_positions(self.group)
-        return lib.attention_positions_per_item(self.group)
+            return lib.attention_prefill_mfma_positions(self.group, key_ways)
+        return lib.attention_positions_per_item(self.group) if key_ways == 1 else 0
+
+    def prefill_key_ways(self, counts) -> int:
+        """1 or 2: how many waves share the keys of a page for the same rows in the prompt
+        step whose sequences bring `counts` tokens.  The matrix-core kernel pairs a long item
+        with a short one per block once there are 512 blocks, which loads every block alike;
+        a step with fewer blocks than that (one prompt of 2,048 tokens of the 8B shape has
+        256, whose walks are 1 to 32 pages long) takes items half as long, and with them
+        twice the blocks."""
+        if not self.matrix_cores or self.positions_per_item(2) == 0:
+            return 1
+        size = self.positions_per_item(1)
+        heads = 4 if self.group % 4 == 0 else (2 if self.group % 2 == 0 else 1)
+        items = sum((count + size - 1) // size for count in counts)
+        blocks = items * (self.group // heads) * self.spec.n_kv_heads
+        return 2 if blocks < 512 else 1
 
     @property
     def plan_key(self):
         """Attention parts with equal keys plan the same sections."""
-        return ("attention", self.positions_per_item())
+        return ("attention", self.positions_per_item(), self.group, self.spec.n_kv_heads)
 
-    def _items_section(self):
-        return f"attention.items{self.positions_per_item()}"
+    def _items_section(self, key_ways: int = 1):
+        return f"attention.items{self.positions_per_item(key_ways)}"
 
     def plan_step(self, plan):
         """The work items of this step's attention kernels, as one int32 section [3, items]:
@@ -137,15 +152,16 @@ class Attention:
         (they take longest, so they start first); a decode step has one item a sequence."""
         if plan.decode:
             return {"attention.decode_items": _decode_items(plan.n_seqs, plan.n_live_seqs)}
-        size = self.positions_per_item()
+        key_ways = self.prefill_key_ways([seq.count for seq in plan.seqs])
+        size = self.positions_per_item(key_ways)
         items = []
         for index, seq in enumerate(plan.seqs):
             for p0 in range(0, seq.count, size):
                 npos = min(size, seq.count - p0)
                 items.append((-(seq.start + p0 + npos), index, seq.row0 + p0, npos))
         items.sort()
-        return {self._items_section(): np.asarray([item[1:] for item in items],
-                                                  dtype=np.int32).T.copy()}
+        return {self._items_section(key_ways): np.asarray([item[1:] for item in items],
+                                                          dtype=np.int32).T.copy()}
 
     @staticmethod
     def _items(ctx, name):
@@ -223,12 +239,14 @@ class Attention:
                               spec.n_kv_heads, spec.head_dim, window=spec.window,
                               scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml)
         else:
-            item_seq, item_row0, item_npos, n_items = self._items(ctx, self._items_section())
+            key_ways = self.prefill_key_ways([seq.count for seq in ctx.sequences])
+            item_seq, item_row0, item_npos, n_items = self._items(
+                ctx, self._items_section(key_ways))
             if self.matrix_cores:
                 lib.attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos,
                                            n_items, meta.row_pos, page_table, out, spec.n_heads,
                                            spec.n_kv_heads, spec.head_dim, window=spec.window,
-                                           scale=self.scale)
+                                           scale=self.scale, key_ways=key_ways)
             else:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,

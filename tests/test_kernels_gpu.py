@@ -291,7 +291,7 @@ def items_for(lib, starts, counts, group, per=None):
 
 
 def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
-                  boost=None, kernel="generic", waves=4, longest=None):
+                  boost=None, kernel="generic", waves=4, longest=None, key_ways=1):
     """Fill a paged cache with random keys and values, run the kernel for the last
     `counts[b]` positions of each sequence, return (kernel output, plain output)."""
     torch.manual_seed(seed)
@@ -316,7 +316,7 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     pos = torch.tensor(row_pos, dtype=torch.int32, device=DEV)
     seq = torch.tensor(row_seq, dtype=torch.int32, device=DEV)
     group = nq // nkv
-    per = lib.attention_prefill_mfma_positions(group) if kernel == "prefill_mfma" else None
+    per = lib.attention_prefill_mfma_positions(group, key_ways) if kernel == "prefill_mfma" else None
     item_seq, item_row0, item_npos, n_items = items_for(lib, starts, counts, group, per)
     out = torch.full((N, nq * D), float("nan"), device=DEV, dtype=dtype)
     part_o = part_ml = None
@@ -326,7 +326,7 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     if kernel == "prefill_mfma":
         lib.attention_prefill_mfma(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0,
                                    item_npos, n_items, pos, cache.table_dev, out, nq, nkv, D,
-                                   window=window)
+                                   window=window, key_ways=key_ways)
     elif kernel == "decode_mfma":
         lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
                                   cache.table_dev, out, nq, nkv, D, window=window,
@@ -517,38 +517,49 @@ def test_attention_decode_from_the_projection(lib, nq, nkv, D, splits, waves, sl
             assert not torch.isnan(kb[page, :, row_pos[r] % PAGE]).any()
 
 
+@pytest.mark.parametrize("key_ways", [1, 2])
 @pytest.mark.parametrize("nq,nkv,D", [(32, 8, 128), (8, 8, 64), (6, 2, 128), (5, 1, 64),
                                       (12, 3, 128), (16, 16, 64), (8, 1, 128), (2, 1, 64)])
-def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D):
+def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D, key_ways):
     """The bfloat16 prefill kernel: prompts of 1, 63, 64, 65 and 300 tokens, and chunks
-    appended to 70 and to 640 cached tokens, in one launch.  Probabilities are rounded to
-    bfloat16 before the value product, which the bound (2^-8 of the largest value) covers."""
+    appended to 70 and to 640 cached tokens, in one launch; every row group with all of a
+    page's keys (key_ways 1) and with two waves sharing them (2: half as many positions an
+    item, the two halves merged at the end).  Probabilities are rounded to bfloat16 before the
+    value product, which the bound (2^-8 of the largest value) covers."""
+    assert lib.attention_prefill_mfma_positions(nq // nkv, 2) * 2 == \
+        lib.attention_prefill_mfma_positions(nq // nkv, 1)
     out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D,
                                   starts=[0, 0, 0, 0, 70, 0, 640],
-                                  counts=[1, 64, 63, 300, 9, 65, 100], kernel="prefill_mfma")
+                                  counts=[1, 64, 63, 300, 9, 65, 100], kernel="prefill_mfma",
+                                  key_ways=key_ways)
     close(out, expected, torch.bfloat16)
 
 
+@pytest.mark.parametrize("key_ways", [1, 2])
 @pytest.mark.parametrize("counts", [[1041, 20], [1060]])
-def test_attention_prefill_on_the_matrix_cores_many_blocks(lib, counts):
+def test_attention_prefill_on_the_matrix_cores_many_blocks(lib, counts, key_ways):
     """Enough work items (more than 512 blocks) for the kernel to give every block two of
     them, the u-th and the u-th from the end; an odd and an even number of items."""
     out, expected = run_attention(lib, torch.bfloat16, 64, 16, 64, starts=[0] * len(counts),
-                                  counts=counts, kernel="prefill_mfma", seed=5)
+                                  counts=counts, kernel="prefill_mfma", seed=5, key_ways=key_ways)
     close(out, expected, torch.bfloat16)
 
 
-@pytest.mark.parametrize("window", [1, 7, 64, 100])
-def test_attention_prefill_on_the_matrix_cores_window_and_far_key(lib, window):
+@pytest.mark.parametrize("key_ways", [1, 2])
+@pytest.mark.parametrize("window", [1, 7, 31, 33, 64, 100])
+def test_attention_prefill_on_the_matrix_cores_window_and_far_key(lib, window, key_ways):
     nq, nkv, D, n = 8, 2, 128, 230
     for key_index in (n - window, n - window - 1):
         out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [0], [n], window=window,
                                       boost=(0, key_index, n - 1, 300.0), seed=9,
-                                      kernel="prefill_mfma")
+                                      kernel="prefill_mfma", key_ways=key_ways)
         close(out, expected, torch.bfloat16)
-    out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [0], [900],
-                                  boost=(0, 3, 899, 200.0), seed=4, kernel="prefill_mfma")
-    close(out, expected, torch.bfloat16)
+    # a far key in the first half of a page and one in the second (keys 3 and 40)
+    for far in (3, 40):
+        out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, [0], [900],
+                                      boost=(0, far, 899, 200.0), seed=4, kernel="prefill_mfma",
+                                      key_ways=key_ways)
+        close(out, expected, torch.bfloat16)
 
 
 def test_attention_refuses_sizes_it_cannot_run(lib):
