@@ -48,7 +48,7 @@ struct DecodePrep {
 
 // GB: query heads of the kv group handled by this block (1..16).  W: waves of the block, each
 // taking every W-th tile of 16 keys of the block's key range: 4 where sequences and slices
-// give many blocks, 16 where they give few (a short range then needs no slices at all).
+// give many blocks, 8 or 16 where they give fewer (a short range then needs no slices at all).
 // PREP: q is not read; the block forms its queries and the position's key and value itself
 // (the block of slice 0 and head block 0 stores them; the wave that meets the position in
 // its tile takes them from LDS, since the store of another block may not have landed).
@@ -868,6 +868,14 @@ void launch_decode(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t*
       return;
     }
   }
+  if constexpr (GB <= 8) {               // and 8 waves at most 8
+    if (waves == 8) {
+      attn_decode_kernel<D, GB, 8, PREP><<<grid, 8 * EI_WAVE, 0, stream>>>(
+          q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
+          head_blocks, window, scale, n_splits, longest, prep);
+      return;
+    }
+  }
   attn_decode_kernel<D, GB, 4, PREP><<<grid, 4 * EI_WAVE, 0, stream>>>(
         q, k, v, row_pos, row_seq, page_table, table_width, out, part_o, part_ml, nq, nkv,
         head_blocks, window, scale, n_splits, longest, prep);
@@ -963,7 +971,8 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
                          float scale, int n_splits, int waves, const int32_t* longest,
                          const DecodePrep* prep, hipStream_t stream) {
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
-  EI_REQUIRE(waves == 4 || waves == 16, "attention_decode: a block has 4 or 16 waves");
+  EI_REQUIRE(waves == 4 || waves == 8 || waves == 16,
+             "attention_decode: a block has 4, 8 or 16 waves");
   EI_REQUIRE(D == 64 || D == 128, "attention_decode: this kernel takes head_dim 64 or 128");
   EI_REQUIRE((q || prep) && k_pages && v_pages && row_pos && row_seq && page_table && out &&
                  table_width > 0,
@@ -972,10 +981,12 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
   EI_REQUIRE(n_splits == 1 || (part_o && part_ml), "attention_decode: split scratch missing");
   EI_REQUIRE(window >= 0, "attention_decode: negative window");
   const int G = nq / nkv;
-  // heads of a kv group that one block takes; blocks of 16 waves take at most 4 (their merge
-  // buffers grow with both), a larger group then has several blocks per kv head
+  // heads of a kv group that one block takes; blocks of 16 waves take at most 4 and blocks of
+  // 8 waves at most 8 (their merge buffers grow with both), a larger group then has several
+  // blocks per kv head
   int GB = G >= 8 ? (G >= 16 ? 16 : 8) : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
   if (waves == 16 && GB > 4) GB = 4;
+  if (waves == 8 && GB > 8) GB = 8;
   const int head_blocks = (G + GB - 1) / GB;
   EI_REQUIRE(static_cast<long long>(nkv) * head_blocks <= 65535, "attention_decode: too many heads");
   dim3 grid(rows, nkv * head_blocks, n_splits);

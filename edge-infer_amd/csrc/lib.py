@@ -366,7 +366,7 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
                           n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
                           part_ml=None, waves=4, longest=None) -> None:
     """bfloat16 decode attention on the matrix cores: one query row per sequence.  `waves`
-    (4 or 16) of a block share its key range tile by tile; 16 suit few sequences (few
+    (4, 8 or 16) of a block share its key range tile by tile; more suit fewer sequences (few
     blocks), whose ranges then need fewer slices or none.  `longest` (int32 [1] on the
     device): the most tokens a sequence of the step holds; every sequence's range is then
     cut into slices of the longest one's share, so that unequal lengths give equal blocks.

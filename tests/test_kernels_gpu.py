@@ -404,11 +404,11 @@ def test_attention_window_edge(lib, dtype, window):
 @pytest.mark.parametrize("nq,nkv,D,splits", [(32, 8, 128, 1), (32, 8, 128, 4), (8, 8, 64, 3), (64, 8, 128, 1),
                                              (6, 2, 128, 2), (20, 1, 64, 5), (16, 1, 128, 32),
                                              (2, 1, 64, 1)])
-@pytest.mark.parametrize("waves", [4, 16])
+@pytest.mark.parametrize("waves", [4, 8, 16])
 def test_attention_decode_on_the_matrix_cores(lib, nq, nkv, D, splits, waves):
     """The bfloat16 decode kernel: lengths around tile (16), page (64) and slice
     boundaries, group ratios that fill a head block partly, more slices than pages; blocks
-    of 4 and of 16 waves (more waves than a short sequence has tiles)."""
+    of 4, 8 and 16 waves (more waves than a short sequence has tiles)."""
     starts = [0, 1, 14, 15, 16, 62, 63, 64, 127, 128, 300, 1029, 8]
     out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, starts=starts,
                                   counts=[1] * len(starts), splits=splits, kernel="decode_mfma",

@@ -1,8 +1,8 @@
 """Contexts of thousands of tokens at head size 128, in float32 and bfloat16, against the
 plain implementation: a long prompt whole; decoding across a context bound, where the
 session moves to another captured graph; a decode batch of very unequal contexts, whose key
-ranges are cut into slices by the longest one; and a batch of so many sequences that
-attention takes its many-blocks launch shape.  The q/k norm weights are raised by half, which
+ranges are cut into slices by the longest one; and batches of so many sequences that
+attention takes its launch shapes of smaller blocks.  The q/k norm weights are raised by half, which
 more than doubles the scores, so that attention is peaked: a key that is left out, read twice
 or read from a foreign page then moves the logits by far more than the tolerance.  (The
 rounding of bfloat16 queries and keys grows with the scores as well: with doubled weights
@@ -157,14 +157,16 @@ def test_a_decode_batch_of_very_unequal_contexts(models, oracle, dtype):
         assert waves == 16 and mixer.decode_launch(1, 300) == (1, 16)
 
 
+@pytest.mark.parametrize("count,waves", [(72, 8), (136, 4)])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_many_sequences_beyond_1024_tokens(models, oracle, dtype):
-    """72 sequences of 1,030 to 1,100 tokens: more (sequence, kv head) pairs than one launch
-    of large blocks takes, so attention runs its many-small-blocks shape at a context where
-    slices matter.  Six of them are compared with the plain implementation, all of them with
-    the same engine running them eight at a time (the other launch shape)."""
+def test_many_sequences_beyond_1024_tokens(models, oracle, dtype, count, waves):
+    """72 and 136 sequences of 1,030 to 1,100 tokens: more (sequence, kv head) pairs than one
+    launch of the largest blocks takes, so attention runs its shapes of 8 and of 4 waves a
+    block at a context where slices matter.  Six of them are compared with the plain
+    implementation, all of them with the same engine running them eight at a time (the
+    16-wave shape)."""
     import edge_infer_amd as ei
-    count, new = 72, 3
+    new = 3
     lengths = [1030 + (37 * i) % 71 for i in range(count)]
     requests = [ids_of(n + new, seed=100 + i) for i, n in enumerate(lengths)]
     model = models(dtype)
@@ -187,10 +189,12 @@ def test_many_sequences_beyond_1024_tokens(models, oracle, dtype):
     wide = ei.Session(model, max_tokens=count * 1152, max_seqs=count, max_seq_tokens=1152)
     got = run(wide, list(range(count)))
     if mixer.matrix_cores:
-        assert mixer.decode_launch(96, 1536)[1] == 4 and mixer.decode_launch(8, 1536)[1] == 16
+        bucket = next(iter(wide._captured))[0]
+        assert mixer.decode_launch(bucket, 1536)[1] == waves
+        assert mixer.decode_launch(8, 1536)[1] == 16
     for r in (0, 1, 17, 40, 70, 71):
         n = lengths[r]
-        assert_close(dtype, got[r], oracle(requests[r])[n - 1:], f"{dtype} request {r} of 72")
+        assert_close(dtype, got[r], oracle(requests[r])[n - 1:], f"{dtype} request {r} of {count}")
     narrow = ei.Session(model, max_tokens=8 * 1152, max_seqs=8, max_seq_tokens=1152)
     bound = 1e-5 if dtype == "float32" else 3e-2
     for first in range(0, count, 8):
