@@ -472,10 +472,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 #pragma unroll
   for (int i = 0; i < CI; ++i) {
     k_write[i] = ld_key * D + place(ld_key, ld_dc + 8 * i) * 8;
-    v_write[i] = ((ld_dc + 8 * i) * 8 + (ld_key & 1)) * VS + (ld_key & ~1);
+    v_write[i] = (ld_dc + 8 * i) * 8 * VS + ld_key;
   }
-  const bool later = ld_dc & 4;
-  const uint32_t take = (ld_key & 1) ? 0x03020706u : 0x05040100u;   // bytes of (partner, own)
 
   for (int pass = 0; pass <= pair; ++pass) {
   const int item = pass == 0 ? unit : n_items - 1 - unit;
@@ -532,6 +530,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
       return;
     }
     const size_t base = ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D + ld_dc * 8;
+    if (page_index < hi_page) {           // a whole page (the same for every lane)
+#pragma unroll
+      for (int i = 0; i < CI; ++i) {
+        k_stage[i] = *reinterpret_cast<const uint4*>(k_pages + base + 64 * i);
+        v_stage[i] = *reinterpret_cast<const uint4*>(v_pages + base + 64 * i);
+      }
+      return;
+    }
     const bool live = page_index * EI_PAGE + ld_key <= last_pos;   // later slots: stale bytes
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
@@ -541,31 +547,21 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
                         : uint4{0u, 0u, 0u, 0u};
     }
   };
-  // Values go to LDS transposed ([d][key]).  A lane holds 8 values of one key as 4 dwords (d
-  // pairs); the lane 8 further in its row of 16 holds the same d of the next key, so after one
-  // exchange (a DPP rotation of the row by 8) the even-key lane owns the two keys of the even d
-  // of every pair and the odd-key lane those of the odd d: 4 dword stores a lane.  The upper 4
-  // lanes of a key take their d pairs one step later, which spreads the stores over the banks.
+  // Values go to LDS transposed ([d][key]): a lane holds 8 values of one key and stores each
+  // as 16 bits at its d row (the row offsets are constants of the instruction, the upper
+  // halves are stored from where they are), which costs no vector arithmetic at all; an
+  // exchange of halves between lanes and dword stores was 50 vector instructions a page more.
   auto store_page = [&](auto buf_tag) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
       *reinterpret_cast<uint4*>(&k_lds[k_write[i] + buf * KBUF]) = k_stage[i];
       const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
-      uint32_t partner[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e)
-        partner[e] = __builtin_amdgcn_update_dpp(0u, w[e], 0x128 /* row_ror:8 */, 0xf, 0xf, false);
-      uint32_t both[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) both[e] = __builtin_amdgcn_perm(partner[e], w[e], take);
-      // d pair e goes to row 2 e (+ the odd key's 1) of the chunk; the later lanes start at pair 1
+      bf16_t* const to = &v_lds[v_write[i] + buf * VBUF];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int e2 = (e + 1) & 3;
-        const uint32_t word = later ? both[e2] : both[e];
-        const int to = v_write[i] + buf * VBUF + (later ? 2 * e2 * VS : 2 * e * VS);
-        *reinterpret_cast<uint32_t*>(&v_lds[to]) = word;
+        to[(2 * e) * VS] = static_cast<bf16_t>(w[e] & 0xffffu);
+        to[(2 * e + 1) * VS] = static_cast<bf16_t>(w[e] >> 16);
       }
     }
   };
