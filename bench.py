@@ -117,17 +117,17 @@ def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True,
     return 1000.0 * elapsed / steps, mean_context, 1000.0 * median
 
 
-def measure_prefill(model, cfg, repeats=3):
+def measure_prefill(model, cfg, repeats=3, tokens=PREFILL_TOKENS):
     import torch
     import edge_infer_amd as ei
-    session = ei.Session(model, max_tokens=PREFILL_TOKENS, max_seqs=1)
-    prompt = synthetic_prompts(cfg, 1, PREFILL_TOKENS, seed=7)[0]
+    session = ei.Session(model, max_tokens=tokens, max_seqs=1)
+    prompt = synthetic_prompts(cfg, 1, tokens, seed=7)[0]
     best = None
     for _ in range(repeats + 1):
         slot = session.begin()
         torch.cuda.synchronize()
         started = time.perf_counter()
-        session.step([(slot, prompt, [PREFILL_TOKENS - 1])], copy=False)
+        session.step([(slot, prompt, [tokens - 1])], copy=False)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - started
         session.end(slot)
@@ -253,6 +253,9 @@ def main():
                         help="tokens a sequence may hold (with --only generate)")
     parser.add_argument("--new-tokens", type=int, default=256,
                         help="tokens generated for each prompt (with --only generate)")
+    parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
+                        help="with --only prefill: the length of the one prompt (the record's "
+                             "prefill is always of 2,048 tokens)")
     parser.add_argument("--with-32b", action="store_true",
                         help="also measure the 32B shape (decode at batch 1 and 16, prefill)")
     parser.add_argument("--peaks", action="store_true",
@@ -296,9 +299,10 @@ def main():
                           "ms_per_decode_step": round(1e3 * (total - prompt_s) / max(1, steps), 4)}))
         return 0
     if args.only == "prefill":
-        prefill_ms = measure_prefill(model, cfg)
-        flops = prefill_flops(cfg, PREFILL_TOKENS)
-        print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": PREFILL_TOKENS,
+        tokens = args.prefill_tokens
+        prefill_ms = measure_prefill(model, cfg, tokens=tokens)
+        flops = prefill_flops(cfg, tokens)
+        print(json.dumps({"only": "prefill", "shape": args.shape, "tokens": tokens,
                           "ms": round(prefill_ms, 3),
                           "TFLOP/s": round(flops / (prefill_ms * 1e-3) / 1e12, 1)}))
         return 0

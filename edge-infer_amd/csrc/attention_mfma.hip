@@ -409,7 +409,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   constexpr int SJ = D / 16;             // 16-wide steps over d for the scores
   constexpr int DB = D / 32;             // 32-wide output blocks over d
   constexpr int VS = EI_PAGE + 4;        // LDS stride of a transposed value row (34 dwords)
-  constexpr int CI = D / 64;             // 16-byte chunks per thread per page
+  constexpr int CI = D / 32;             // 16-byte chunks per thread per page
   constexpr int CHUNKS = D / 8;          // 16-byte chunks of a key row
   constexpr int KBUF = EI_PAGE * D, VBUF = D * VS;    // elements of one page buffer
   constexpr int NG = kPrefillWaves / (HB * KW);       // groups of 32 rows in a block
@@ -467,13 +467,15 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 #pragma unroll
   for (int sj = 0; sj < SJ; ++sj) k_read[sj] = n32 * D + place(n32, 2 * sj + half) * 8;
   const int v_read = n32 * VS + 4 * half;
-  const int ld_key = t >> 3, ld_dc = t & 7;
-  int k_write[CI], v_write[CI];
+  // waves 0..3 move the page's keys, waves 4..7 its values: four lanes a row, chunks
+  // ld_dc + 4 i of it.  (With eight lanes a row the 16-bit stores of the values' transposition
+  // met every bank twice: rows 32 apart lie 16 banks apart four times over.)
+  const bool moves_values = t >= kPrefillThreads / 2;
+  const int ld_key = (t & (kPrefillThreads / 2 - 1)) >> 2, ld_dc = t & 3;
+  int k_write[CI];
 #pragma unroll
-  for (int i = 0; i < CI; ++i) {
-    k_write[i] = ld_key * D + place(ld_key, ld_dc + 8 * i) * 8;
-    v_write[i] = (ld_dc + 8 * i) * 8 * VS + ld_key;
-  }
+  for (int i = 0; i < CI; ++i) k_write[i] = ld_key * D + place(ld_key, ld_dc + 4 * i) * 8;
+  const int v_write = ld_dc * 8 * VS + ld_key;
 
   for (int pass = 0; pass <= pair; ++pass) {
   const int item = pass == 0 ? unit : n_items - 1 - unit;
@@ -518,7 +520,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[db][e] = 0.f;
 
-  uint4 k_stage[CI], v_stage[CI];
+  uint4 stage[CI];
   auto lookup = [&](int page_index) __attribute__((always_inline)) {
     return page_index <= hi_page
                ? page_table[static_cast<size_t>(seq) * table_width + page_index] : -1;
@@ -526,26 +528,21 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   auto load_page = [&](int page_index, int phys) __attribute__((always_inline)) {
     if (phys < 0) {                       // released by the window: every key is masked
 #pragma unroll
-      for (int i = 0; i < CI; ++i) k_stage[i] = v_stage[i] = uint4{0u, 0u, 0u, 0u};
+      for (int i = 0; i < CI; ++i) stage[i] = uint4{0u, 0u, 0u, 0u};
       return;
     }
-    const size_t base = ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D + ld_dc * 8;
+    const bf16_t* const src =
+        (moves_values ? v_pages : k_pages) +
+        ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D + ld_dc * 8;
     if (page_index < hi_page) {           // a whole page (the same for every lane)
 #pragma unroll
-      for (int i = 0; i < CI; ++i) {
-        k_stage[i] = *reinterpret_cast<const uint4*>(k_pages + base + 64 * i);
-        v_stage[i] = *reinterpret_cast<const uint4*>(v_pages + base + 64 * i);
-      }
+      for (int i = 0; i < CI; ++i) stage[i] = *reinterpret_cast<const uint4*>(src + 32 * i);
       return;
     }
     const bool live = page_index * EI_PAGE + ld_key <= last_pos;   // later slots: stale bytes
 #pragma unroll
-    for (int i = 0; i < CI; ++i) {
-      k_stage[i] = live ? *reinterpret_cast<const uint4*>(k_pages + base + 64 * i)
-                        : uint4{0u, 0u, 0u, 0u};
-      v_stage[i] = live ? *reinterpret_cast<const uint4*>(v_pages + base + 64 * i)
-                        : uint4{0u, 0u, 0u, 0u};
-    }
+    for (int i = 0; i < CI; ++i)
+      stage[i] = live ? *reinterpret_cast<const uint4*>(src + 32 * i) : uint4{0u, 0u, 0u, 0u};
   };
   // Values go to LDS transposed ([d][key]): a lane holds 8 values of one key and stores each
   // as 16 bits at its d row (the row offsets are constants of the instruction, the upper
@@ -553,11 +550,16 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   // exchange of halves between lanes and dword stores was 50 vector instructions a page more.
   auto store_page = [&](auto buf_tag) __attribute__((always_inline)) {
     constexpr int buf = decltype(buf_tag)::value;
+    if (!moves_values) {
+#pragma unroll
+      for (int i = 0; i < CI; ++i)
+        *reinterpret_cast<uint4*>(&k_lds[k_write[i] + buf * KBUF]) = stage[i];
+      return;
+    }
 #pragma unroll
     for (int i = 0; i < CI; ++i) {
-      *reinterpret_cast<uint4*>(&k_lds[k_write[i] + buf * KBUF]) = k_stage[i];
-      const uint32_t w[4] = {v_stage[i].x, v_stage[i].y, v_stage[i].z, v_stage[i].w};
-      bf16_t* const to = &v_lds[v_write[i] + buf * VBUF];
+      const uint32_t w[4] = {stage[i].x, stage[i].y, stage[i].z, stage[i].w};
+      bf16_t* const to = &v_lds[v_write + buf * VBUF + 4 * i * 8 * VS];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         to[(2 * e) * VS] = static_cast<bf16_t>(w[e] & 0xffffu);
