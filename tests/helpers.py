@@ -5,12 +5,19 @@ from pathlib import Path
 import torch
 
 # float32 engine against the float64 plain implementation, relative to the largest logit
-F32_REL = 1e-4
+# (the largest seen in the whole suite is 4.7e-6, on a layer of the 8B widths)
+F32_REL = 2e-5
 # bfloat16 engine against the plain implementation: root-mean-square and maximum error
 # relative to the root-mean-square and the maximum logit (bfloat16 keeps 8 significant
-# bits, 2^-9 relative per rounding; a few dozen roundings accumulate per token)
-BF16_RMS_REL = 2e-2
-BF16_MAX_REL = 6e-2
+# bits, 2^-9 relative per rounding; a few dozen roundings accumulate per token).  The largest
+# seen: 0.6 % / 0.75 % on the tiny models, 0.86 % / 0.91 % on a layer of the 8B widths.
+BF16_RMS_REL = 1.2e-2
+BF16_MAX_REL = 1.5e-2
+# the same for the tests of thousands of tokens with raised q/k norm weights, whose scores
+# (and with them the rounding of bfloat16 queries and keys) are more than twice as large:
+# 1.46 % / 2.03 % seen
+BF16_LONG_RMS_REL = 2e-2
+BF16_LONG_MAX_REL = 3e-2
 
 TINY_A = dict(vocab_size=256, hidden_size=64, num_hidden_layers=2, num_attention_heads=4,
               num_key_value_heads=2, head_dim=16, intermediate_size=128,
@@ -42,26 +49,47 @@ def random_ids(vocab, count, seed):
     return torch.randint(0, vocab, (count,), generator=g).tolist()
 
 
+_SEEN = {}
+
+
+def _record(kind, value, what):
+    import os
+    path = os.environ.get("EI_TEST_RECORD_ERRORS")
+    if path and value > _SEEN.get(kind, (0.0, ""))[0]:
+        _SEEN[kind] = (value, what)
+        with open(path, "a") as out:
+            out.write(f"{kind} {value:.3e} {what}\n")
+
+
 def assert_close_f32(actual, expected, what=""):
     actual, expected = actual.double().cpu(), expected.double().cpu()
     scale = expected.abs().max().item()
     err = (actual - expected).abs().max().item()
+    _record("f32", err / scale, what)
     assert err <= F32_REL * scale, f"{what}: max error {err:.3e} against scale {scale:.3e}"
 
 
-def assert_close_bf16(actual, expected, what=""):
+def assert_close_bf16(actual, expected, what="", rms_rel=BF16_RMS_REL, max_rel=BF16_MAX_REL):
     actual, expected = actual.double().cpu(), expected.double().cpu()
     diff = actual - expected
     rms = diff.pow(2).mean().sqrt().item()
     ref_rms = expected.pow(2).mean().sqrt().item()
     worst = diff.abs().max().item()
     scale = expected.abs().max().item()
-    assert rms <= BF16_RMS_REL * ref_rms, f"{what}: rms error {rms:.3e} against {ref_rms:.3e}"
-    assert worst <= BF16_MAX_REL * scale, f"{what}: max error {worst:.3e} against {scale:.3e}"
+    _record("bf16_rms", rms / ref_rms, what)
+    _record("bf16_max", worst / scale, what)
+    assert rms <= rms_rel * ref_rms, f"{what}: rms error {rms:.3e} against {ref_rms:.3e}"
+    assert worst <= max_rel * scale, f"{what}: max error {worst:.3e} against {scale:.3e}"
 
 
-def assert_close(dtype, actual, expected, what=""):
+def assert_close(dtype, actual, expected, what="", **bf16_bounds):
     if dtype == "float32":
         assert_close_f32(actual, expected, what)
     else:
-        assert_close_bf16(actual, expected, what)
+        assert_close_bf16(actual, expected, what, **bf16_bounds)
+
+
+def assert_close_long(dtype, actual, expected, what=""):
+    """For the long-context models with raised q/k norm weights."""
+    assert_close(dtype, actual, expected, what, rms_rel=BF16_LONG_RMS_REL,
+                 max_rel=BF16_LONG_MAX_REL)

@@ -312,7 +312,7 @@ def test_greedy_generation_through_the_entry_point(folders, oracle, name, dtype)
             if agree < len(expected):
                 logits = plain.forward(w, cfg, prompt + expected[:agree])[-1]
                 gap = (logits[expected[agree]] - logits[got[i][agree]]).item()
-                assert 0 <= gap <= 0.06 * logits.abs().max().item(), f"request {i} step {agree}"
+                assert 0 <= gap <= 0.03 * logits.abs().max().item(), f"request {i} step {agree}"
         assert [t for j, t in seen if j == i] == got[i]
     # the single-request call of the reference's API: max_length counts the prompt
     single = session.generate(prompts[1], max_length=len(prompts[1]) + 4, top_k=1)
@@ -329,7 +329,7 @@ def test_greedy_generation_through_the_entry_point(folders, oracle, name, dtype)
             assert agree < len(single), "the request ended early"
             logits = plain.forward(w, cfg, prompts[1] + first4[:agree])[-1]
             gap = (logits[first4[agree]] - logits[single[agree]]).item()
-            assert 0 <= gap <= 0.06 * logits.abs().max().item(), f"alone, step {agree}"
+            assert 0 <= gap <= 0.03 * logits.abs().max().item(), f"alone, step {agree}"
     assert session.generate(prompts[1], max_length=len(prompts[1])) == []
     # the end-of-sequence token ends a request and is not delivered
     if dtype == "float32":

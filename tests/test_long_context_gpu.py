@@ -11,7 +11,7 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
-from helpers import assert_close, random_ids
+from helpers import assert_close_long as assert_close, random_ids
 
 pytestmark = pytest.mark.gpu
 
