@@ -312,12 +312,18 @@ def attention_decode_mfma_supported(head_dim: int, group: int) -> bool:
     return head_dim in MFMA_HEAD_DIMS and group >= 1
 
 
+def attention_prefill_mfma_heads(group: int) -> int:
+    """Query heads of a kv group that one block of the matrix-core prefill kernel takes: the
+    largest of 4, 2, 1 that divides the group."""
+    return 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
+
+
 def attention_prefill_mfma_positions(group: int, key_ways: int = 1) -> int:
     """Positions of a sequence per work item of the matrix-core prefill kernel: a block of 8
     waves holds 4, 2 or 1 heads of a kv group, each wave 32 positions of one head; with
     `key_ways` = 2 two waves share the keys of every page for the same positions, so an item
     is half as long (0: the group has no such form)."""
-    heads = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
+    heads = attention_prefill_mfma_heads(group)
     if key_ways not in (1, 2) or heads * key_ways > 8:
         return 0
     return 32 * (8 // (heads * key_ways))

@@ -132,7 +132,7 @@ class Attention:
         if not self.matrix_cores or self.positions_per_item(2) == 0:
             return 1
         size = self.positions_per_item(1)
-        heads = 4 if self.group % 4 == 0 else (2 if self.group % 2 == 0 else 1)
+        heads = lib.attention_prefill_mfma_heads(self.group)
         items = sum((count + size - 1) // size for count in counts)
         blocks = items * (self.group // heads) * self.spec.n_kv_heads
         return 2 if blocks < 512 else 1
