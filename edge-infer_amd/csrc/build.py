@@ -120,9 +120,17 @@ def build_library(name: str, force: bool = False, quiet: bool = False) -> Path:
     return target
 
 
-def build_all(force: bool = True, jobs: int = 8) -> None:
-    names = available_libraries()
+def build_libraries(names, force: bool = False, jobs: int = 8) -> None:
+    """Compile those of `names` that are not built yet (all of them with `force`), side by
+    side: what a model needs is then ready after the longest compilation, not their sum."""
+    names = [name for name in dict.fromkeys(names) if force or not is_current(name)]
+    if not names:
+        return
     _build_dir()
     with ThreadPoolExecutor(max_workers=max(1, min(jobs, len(names)))) as pool:
         for _ in pool.map(lambda n: build_library(n, force=force), names):
             pass
+
+
+def build_all(force: bool = True, jobs: int = 8) -> None:
+    build_libraries(available_libraries(), force=force, jobs=jobs)

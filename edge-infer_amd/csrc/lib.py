@@ -115,6 +115,12 @@ def loaded_libraries():
     return sorted(_loaded)
 
 
+def prepare(names) -> None:
+    """Compile the kernel libraries `names` that are not built yet, at the same time.  A
+    model says which ones it will need when it is made; each is still loaded at its first use."""
+    build.build_libraries([name for name in names if name not in _loaded])
+
+
 def _check(lib, status: int, what: str) -> None:
     if status != 0:
         message = lib.ei_last_error().decode(errors="replace")

@@ -116,6 +116,7 @@ class DecoderModel:
         if missing:
             raise KeyError(f"model parameters missing: {missing}")
         self._positions = {}
+        lib.prepare(self.kernel_libraries(spec, self.dtype))
         self.embed = params["embed.weight"].to(device=self.device, dtype=self.dtype).contiguous()
         self.layers = []
         for index, layer in enumerate(spec.layers):
@@ -134,6 +135,19 @@ class DecoderModel:
                                bias=params.get("head.bias"))
         else:  # tied: the head is the embedding table itself (no copy: same type and device)
             self.head = Linear(self.embed, self.dtype, self.device, bias=params.get("head.bias"))
+
+    @staticmethod
+    def kernel_libraries(spec: ModelSpec, dtype):
+        """The kernel libraries a model of `spec` will run, as its parts' classes tell
+        (`kernel_libraries(spec, dtype)`, optional): they are compiled side by side before the
+        model is made, where they are not built yet, instead of one after the other at their
+        first use."""
+        names = ["rowwise", *Linear.kernel_libraries(dtype)]        # embedding, norms, head
+        for layer in spec.layers:
+            ask = getattr(lookup("block", layer.block), "kernel_libraries", None)
+            if ask is not None:
+                names.extend(ask(layer, dtype))
+        return tuple(dict.fromkeys(names))
 
     def position_table(self, position_spec):
         """One shared encoding object per distinct position spec."""

@@ -79,6 +79,15 @@ class Attention:
         return KVRequest(n_kv_heads=spec.n_kv_heads, head_dim=spec.head_dim, window=spec.window)
 
     @classmethod
+    def kernel_libraries(cls, spec, dtype):
+        """What this part will run, so that a model can have it compiled ahead of its first
+        step."""
+        group = spec.n_heads // max(1, spec.n_kv_heads)
+        fast = dtype == torch.bfloat16 and lib.attention_decode_mfma_supported(spec.head_dim, group)
+        return ("rope_store", "attention_mfma" if fast else "attention_generic",
+                *Linear.kernel_libraries(dtype))
+
+    @classmethod
     def check(cls, spec):
         if spec.n_heads % spec.n_kv_heads:
             raise ValueError("attention: n_heads must be a multiple of n_kv_heads")

@@ -35,6 +35,17 @@ class PreNormBlock:
     def mixer_spec(cls, layer_spec):
         return layer_spec.mixer
 
+    @classmethod
+    def kernel_libraries(cls, layer_spec, dtype):
+        """The kernel libraries its parts say they run (a part without the method says none)."""
+        names = []
+        for category, spec in (("norm", layer_spec.norm), ("mixer", layer_spec.mixer),
+                               ("feed_forward", layer_spec.feed_forward)):
+            ask = getattr(lookup(category, spec.kind), "kernel_libraries", None)
+            if ask is not None:
+                names.extend(ask(spec, dtype))
+        return tuple(names)
+
     def __init__(self, layer_spec, hidden, params, dtype, device, positions):
         def sub(prefix):
             return {name[len(prefix) + 1:]: tensor for name, tensor in params.items()

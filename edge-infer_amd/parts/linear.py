@@ -36,6 +36,11 @@ GATED_UNSLICED_BYTES = 200 * 1000 * 1000
 
 
 class Linear:
+    @staticmethod
+    def kernel_libraries(dtype):
+        """The kernel libraries a product in `dtype` runs."""
+        return ("gemm_bf16", "rowwise") if dtype == torch.bfloat16 else ("gemm_f32", "rowwise")
+
     def __init__(self, weight: torch.Tensor, dtype, device, bias: torch.Tensor = None):
         if weight.dim() != 2:
             raise ValueError("a linear weight must be a matrix [out, in]")

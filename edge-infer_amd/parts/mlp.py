@@ -28,6 +28,10 @@ class GatedMLP:
         return min(self.gate_up.capture_rows, self.down.capture_rows)
 
     @classmethod
+    def kernel_libraries(cls, spec, dtype):
+        return ("rowwise", *Linear.kernel_libraries(dtype))
+
+    @classmethod
     def parameters(cls, spec, hidden):
         return {
             "gate_proj.weight": ParamSpec((spec.intermediate_size, hidden)),

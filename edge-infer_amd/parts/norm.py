@@ -17,6 +17,10 @@ class RMSNorm:
     capture_safe = True      # only capturable kernels, no allocation per step
 
     @classmethod
+    def kernel_libraries(cls, spec, dtype):
+        return ("rowwise",)
+
+    @classmethod
     def parameters(cls, spec, width):
         return {"weight": ParamSpec((width,), init="norm")}
 

@@ -125,3 +125,36 @@ def test_checkpoint_names():
     assert name("head.weight") == "lm_head.weight"
     with pytest.raises(KeyError):
         name("layers.0.mixer.gate.weight")
+
+
+def test_a_model_names_the_kernel_libraries_it_will_run():
+    """What is compiled at a model's first use is what that model needs: head sizes 64 and 128
+    in bfloat16 take the matrix-core attention library, everything else the generic one, and a
+    part that says nothing (a toy part of a test) asks for nothing."""
+    import torch
+    from edge_infer_amd import Qwen3Config
+    from edge_infer_amd.engine.model import DecoderModel
+    from edge_infer_amd.parts import register_mixer, unregister
+    from helpers import TINY_A
+
+    small = Qwen3Config(**TINY_A).model_spec()                       # head_dim 16
+    wide = Qwen3Config(**{**TINY_A, "head_dim": 128}).model_spec()
+    assert set(DecoderModel.kernel_libraries(small, torch.float32)) == \
+        {"rowwise", "gemm_f32", "rope_store", "attention_generic"}
+    assert set(DecoderModel.kernel_libraries(small, torch.bfloat16)) == \
+        {"rowwise", "gemm_bf16", "rope_store", "attention_generic"}
+    assert set(DecoderModel.kernel_libraries(wide, torch.bfloat16)) == \
+        {"rowwise", "gemm_bf16", "rope_store", "attention_mfma"}
+    assert "attention_mfma" not in DecoderModel.kernel_libraries(wide, torch.float32)
+
+    class Silent:            # no kernel_libraries
+        pass
+    register_mixer("toy_silent", Silent)
+    try:
+        import dataclasses
+        layer = dataclasses.replace(small.layers[0],
+                                    mixer=dataclasses.replace(small.layers[0].mixer, kind="toy_silent"))
+        toy = dataclasses.replace(small, layers=(layer,) * len(small.layers))
+        assert "attention_generic" not in DecoderModel.kernel_libraries(toy, torch.float32)
+    finally:
+        unregister("mixer", "toy_silent")
