@@ -130,3 +130,13 @@ def test_procedural_interface_without_a_model(capsys):
     assert api.is_cuda_available() == api.is_gpu_available()
     import inspect
     assert inspect.signature(api.generate_text_stream).parameters["top_k"].default == 50
+
+
+def test_the_measurement_program_runs_on_one_gpu_only():
+    """bench.py keeps its contract at one GPU; asked for more it says so in one line and
+    exits with 2, before it touches any device."""
+    root = Path(__file__).resolve().parent.parent
+    done = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"],
+                          capture_output=True, text=True, timeout=120)
+    assert done.returncode == 2
+    assert len(done.stdout.strip().splitlines()) == 1 and "one GPU" in done.stdout
