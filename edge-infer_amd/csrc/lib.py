@@ -49,7 +49,7 @@ _SIGNATURES = {
         "ei_attn_prefill_mfma_positions": [c_int],
         "ei_attention_prefill_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                       c_int, c_void_p, c_void_p, c_int, c_void_p, c_int, c_int,
-                                      c_int, c_int, c_float, c_int, c_void_p],
+                                      c_int, c_int, c_float, c_int, c_int, c_void_p],
         "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
                                      c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
@@ -337,9 +337,11 @@ def attention_prefill_mfma_positions(group: int, key_ways: int = 1) -> int:
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                            page_table, out, n_heads, n_kv_heads, head_dim, window=None,
-                           scale=None, key_ways=1) -> None:
+                           scale=None, key_ways=1, pair_items=True) -> None:
     """bfloat16 prefill attention on the matrix cores; an item holds up to
-    `attention_prefill_mfma_positions(group, key_ways)` positions of one sequence."""
+    `attention_prefill_mfma_positions(group, key_ways)` positions of one sequence.
+    pair_items: with enough items a block may take item i and then item n_items - 1 - i
+    (equal work a block where the items are those of one prompt, longest first)."""
     lib = library("attention_mfma")
     n = q.shape[0]
     if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
@@ -358,7 +360,7 @@ def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, 
         n_items, _gpu(row_pos, "row_pos", torch.int32),
         _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
         _gpu(out, "out", torch.bfloat16), n_heads, n_kv_heads, head_dim, int(window or 0),
-        float(scale), int(key_ways), _stream())
+        float(scale), int(key_ways), int(bool(pair_items)), _stream())
     _check(lib, status, "attention_prefill")
 
 

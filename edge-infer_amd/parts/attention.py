@@ -261,7 +261,8 @@ class Attention:
                 lib.attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos,
                                            n_items, meta.row_pos, page_table, out, spec.n_heads,
                                            spec.n_kv_heads, spec.head_dim, window=spec.window,
-                                           scale=self.scale, key_ways=key_ways)
+                                           scale=self.scale, key_ways=key_ways,
+                                           pair_items=len({(seq.start, seq.count) for seq in ctx.sequences}) == 1)
             else:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,

@@ -291,7 +291,8 @@ def items_for(lib, starts, counts, group, per=None):
 
 
 def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
-                  boost=None, kernel="generic", waves=4, longest=None, key_ways=1):
+                  boost=None, kernel="generic", waves=4, longest=None, key_ways=1,
+                  pair_items=True):
     """Fill a paged cache with random keys and values, run the kernel for the last
     `counts[b]` positions of each sequence, return (kernel output, plain output)."""
     torch.manual_seed(seed)
@@ -326,7 +327,7 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
     if kernel == "prefill_mfma":
         lib.attention_prefill_mfma(q.reshape(N, nq * D), cache.k, cache.v, item_seq, item_row0,
                                    item_npos, n_items, pos, cache.table_dev, out, nq, nkv, D,
-                                   window=window, key_ways=key_ways)
+                                   window=window, key_ways=key_ways, pair_items=pair_items)
     elif kernel == "decode_mfma":
         lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
                                   cache.table_dev, out, nq, nkv, D, window=window,
@@ -535,13 +536,16 @@ def test_attention_prefill_on_the_matrix_cores(lib, nq, nkv, D, key_ways):
     close(out, expected, torch.bfloat16)
 
 
+@pytest.mark.parametrize("pair_items", [True, False])
 @pytest.mark.parametrize("key_ways", [1, 2])
 @pytest.mark.parametrize("counts", [[1041, 20], [1060]])
-def test_attention_prefill_on_the_matrix_cores_many_blocks(lib, counts, key_ways):
+def test_attention_prefill_on_the_matrix_cores_many_blocks(lib, counts, key_ways, pair_items):
     """Enough work items (more than 512 blocks) for the kernel to give every block two of
-    them, the u-th and the u-th from the end; an odd and an even number of items."""
+    them, the u-th and the u-th from the end, where the caller allows it; an odd and an even
+    number of items.  The same items one a block give the same result."""
     out, expected = run_attention(lib, torch.bfloat16, 64, 16, 64, starts=[0] * len(counts),
-                                  counts=counts, kernel="prefill_mfma", seed=5, key_ways=key_ways)
+                                  counts=counts, kernel="prefill_mfma", seed=5, key_ways=key_ways,
+                                  pair_items=pair_items)
     close(out, expected, torch.bfloat16)
 
 
