@@ -980,7 +980,7 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
                          const int32_t* row_pos, const int32_t* row_seq,
                          const int32_t* page_table, int table_width, void* out, float* part_o,
                          float* part_ml, int rows, int nq, int nkv, int D, int window,
-                         float scale, int n_splits, int waves, const int32_t* longest,
+                         float scale, int n_splits, int waves, int heads, const int32_t* longest,
                          const DecodePrep* prep, hipStream_t stream) {
   EI_REQUIRE(rows > 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention_decode: bad head counts");
   EI_REQUIRE(waves == 4 || waves == 8 || waves == 16,
@@ -999,6 +999,12 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
   int GB = G >= 8 ? (G >= 16 ? 16 : 8) : (G >= 4 ? 4 : (G >= 2 ? 2 : 1));
   if (waves == 16 && GB > 4) GB = 4;
   if (waves == 8 && GB > 8) GB = 8;
+  // the caller may ask for fewer (a power of two): more, lighter blocks where the step has
+  // too few of them to occupy the chip
+  if (heads > 0) {
+    EI_REQUIRE((heads & (heads - 1)) == 0, "attention_decode: heads a block must be a power of two");
+    if (heads < GB) GB = heads;
+  }
   const int head_blocks = (G + GB - 1) / GB;
   EI_REQUIRE(static_cast<long long>(nkv) * head_blocks <= 65535, "attention_decode: too many heads");
   dim3 grid(rows, nkv * head_blocks, n_splits);
@@ -1052,15 +1058,19 @@ static int decode_launch(const void* q, const void* k_pages, const void* v_pages
 // pages: [n_pages, nkv, 64, D]; n_splits > 1 needs part_o [rows, nq, n_splits, D] and
 // part_ml [rows, nq, n_splits, 2] float32.  longest (or null): one int32 on the device, the most
 // tokens that a sequence of this step holds; slices are then that sequence's share for all.
+// heads: query heads of a kv group that one block takes (a power of two; 0: as many as a
+// block of `waves` waves can, 4 for 16 waves, 8 for 8, else 16); a group of more has several
+// blocks.
 extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, const void* v_pages,
                                         const int32_t* row_pos, const int32_t* row_seq,
                                         const int32_t* page_table, int table_width, void* out,
                                         float* part_o, float* part_ml, int rows, int nq, int nkv,
                                         int D, int window, float scale, int n_splits,
-                                        int waves, const int32_t* longest, hipStream_t stream) {
+                                        int waves, int heads, const int32_t* longest,
+                                        hipStream_t stream) {
   return decode_launch(q, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
-                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, longest,
-                       nullptr, stream);
+                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, heads,
+                       longest, nullptr, stream);
 }
 
 // The same from the fused projection instead of q: qkv float32 [nsplit][rows, (nq + 2 nkv) * D]
@@ -1073,7 +1083,7 @@ extern "C" int ei_attention_decode_mfma_fused(
     const float* k_norm_w, float eps, const float* rope_table, int write_cache, void* k_pages,
     void* v_pages, const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table,
     int table_width, void* out, float* part_o, float* part_ml, int rows, int nq, int nkv, int D,
-    int window, float scale, int n_splits, int waves, const int32_t* longest,
+    int window, float scale, int n_splits, int waves, int heads, const int32_t* longest,
     hipStream_t stream) {
   EI_REQUIRE(qkv && nsplit >= 1 && split_stride >= 0, "attention_decode_fused: bad projection");
   DecodePrep prep{};
@@ -1087,6 +1097,6 @@ extern "C" int ei_attention_decode_mfma_fused(
   prep.k_store = write_cache ? static_cast<bf16_t*>(k_pages) : nullptr;
   prep.v_store = write_cache ? static_cast<bf16_t*>(v_pages) : nullptr;
   return decode_launch(nullptr, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,
-                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, longest,
-                       &prep, stream);
+                       part_o, part_ml, rows, nq, nkv, D, window, scale, n_splits, waves, heads,
+                       longest, &prep, stream);
 }

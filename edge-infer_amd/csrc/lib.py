@@ -52,12 +52,13 @@ _SIGNATURES = {
                                       c_int, c_int, c_float, c_int, c_int, c_void_p],
         "ei_attention_decode_mfma": [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                      c_int, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
-                                     c_int, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
+                                     c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
+                                     c_void_p],
         "ei_attention_decode_mfma_fused": [c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_float,
                                            c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                            c_int, c_int, c_int, c_int, c_float, c_int, c_int,
-                                           c_void_p, c_void_p],
+                                           c_int, c_void_p, c_void_p],
     },
     "gemm_f32": {
         "ei_gemm_f32": [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_longlong, c_longlong,
@@ -378,10 +379,12 @@ class DecodeProjection:
 
 def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out, n_heads,
                           n_kv_heads, head_dim, window=None, scale=None, n_splits=1, part_o=None,
-                          part_ml=None, waves=4, longest=None) -> None:
+                          part_ml=None, waves=4, longest=None, heads=0) -> None:
     """bfloat16 decode attention on the matrix cores: one query row per sequence.  `waves`
     (4, 8 or 16) of a block share its key range tile by tile; more suit fewer sequences (few
-    blocks), whose ranges then need fewer slices or none.  `longest` (int32 [1] on the
+    blocks), whose ranges then need fewer slices or none.  `heads` (a power of two, or 0 for
+    as many as the block size allows): query heads of a kv group that one block takes; fewer
+    give more, lighter blocks.  `longest` (int32 [1] on the
     device): the most tokens a sequence of the step holds; every sequence's range is then
     cut into slices of the longest one's share, so that unequal lengths give equal blocks.
     `q` is the queries [rows, heads * head_dim], or a `DecodeProjection`: the kernel then does
@@ -428,7 +431,8 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
             None if part_o is None else _gpu(part_o, "part_o", torch.float32),
             None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
             n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves),
-            None if longest is None else _gpu(longest, "longest", torch.int32), _stream())
+            int(heads), None if longest is None else _gpu(longest, "longest", torch.int32),
+            _stream())
         _check(lib, status, "attention_decode")
         return
     status = lib.ei_attention_decode_mfma(
@@ -438,7 +442,7 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
         page_table.shape[-1], _gpu(out, "out", torch.bfloat16),
         None if part_o is None else _gpu(part_o, "part_o", torch.float32),
         None if part_ml is None else _gpu(part_ml, "part_ml", torch.float32), n, n_heads,
-        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves),
+        n_kv_heads, head_dim, int(window or 0), float(scale), n_splits, int(waves), int(heads),
         None if longest is None else _gpu(longest, "longest", torch.int32), _stream())
     _check(lib, status, "attention_decode")
 

@@ -30,7 +30,8 @@ FUSED_DECODE = os.environ.get("EDGE_INFER_FUSED_DECODE", "1") != "0"
 # What the matrix-core decode kernel costs, measured on an MI355X (head size 128): a wave
 # walks a tile of 16 keys in 1.9 us; merging slices costs 4.5 us and 0.1 us a slice.
 TILE_US, MERGE_US, MERGE_SLICE_US = 1.9, 4.5, 0.1
-WAVE_SLOTS = 256 * 16         # waves the chip holds at once: compute units x waves a unit
+COMPUTE_UNITS = 256
+WAVE_SLOTS = COMPUTE_UNITS * 16     # waves the chip holds at once: compute units x waves a unit
 MAX_SLICES = 32
 
 
@@ -179,15 +180,19 @@ class Attention:
         return section[:count], section[count:2 * count], section[2 * count:], count
 
     def decode_launch(self, n_seqs: int, context: int):
-        """(slices of the key range, waves a block) of a decode step over `n_seqs` sequences
-        of up to `context` tokens.  A slice is the same number of pages for every sequence.
+        """(slices of the key range, waves a block, query heads of a group a block takes) of
+        a decode step over `n_seqs` sequences of up to `context` tokens.  A slice is the same
+        number of pages for every sequence.
 
         Matrix-core kernel, up to 256 (sequence, kv head) pairs: blocks of 16 waves, a tile
         of 16 keys per wave at a time, and as many slices as shorten a wave's walk by more
-        than the merge kernel costs, while all blocks still fit the chip at once.  Up to 512
-        pairs: blocks of 8 waves, no slices.  More pairs, and the generic kernel: blocks of 4
-        waves and enough slices to put about two blocks on each of the 256 compute units,
-        never more than there are pages."""
+        than the merge kernel costs, while all blocks still fit the chip at once; if they
+        then leave compute units empty, a block takes fewer heads (2 or 1 instead of 4), as
+        long as every block still has a unit of its own: the keys are fetched once more per
+        block, from the L2, and each block has less to do per tile.  Up to 512 pairs: blocks
+        of 8 waves, no slices.  More pairs, and the generic kernel: blocks of 4 waves and
+        enough slices to put about two blocks on each of the 256 compute units, never more
+        than there are pages."""
         pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
         n_kv_heads = self.spec.n_kv_heads
         if self.matrix_cores:
@@ -204,15 +209,21 @@ class Attention:
                     if cost < best_cost:
                         best, best_cost = slices, cost
                     slices *= 2
-                return best, 16
+                heads = min(4, 1 << (self.group.bit_length() - 1))
+                while heads > 1:
+                    blocks = n_seqs * n_kv_heads * best * -(-self.group // (heads // 2))
+                    if blocks > COMPUTE_UNITS:
+                        break
+                    heads //= 2
+                return best, 16, heads
             # up to 512 pairs of at most 8 heads: blocks of 8 waves fill the chip's wave slots
             # once without slices (measured 1 to 3 % ahead of 4 waves at 32 to 64 sequences)
             pairs = n_seqs * n_kv_heads * ((self.group + 7) // 8)
             if pairs <= 512:
-                return 1, 8
+                return 1, 8, 0
         blocks = n_seqs * n_kv_heads
         wanted = (512 + blocks - 1) // blocks
-        return max(1, min(wanted, pages, MAX_SLICES)), 4
+        return max(1, min(wanted, pages, MAX_SLICES)), 4, 0
 
     def forward(self, ctx, x, entry):
         spec = self.spec
@@ -235,7 +246,7 @@ class Attention:
         out = ctx.buffer("attn.out", (n, spec.q_width))
         part_o = part_ml = None
         if ctx.decode:
-            splits, waves = self.decode_launch(ctx.n_seqs, ctx.context_bound)
+            splits, waves, heads = self.decode_launch(ctx.n_seqs, ctx.context_bound)
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
                                     torch.float32)
@@ -246,7 +257,7 @@ class Attention:
                                           page_table, out, spec.n_heads, spec.n_kv_heads,
                                           spec.head_dim, window=spec.window, scale=self.scale,
                                           n_splits=splits, part_o=part_o, part_ml=part_ml,
-                                          waves=waves, longest=meta.longest)
+                                          waves=waves, longest=meta.longest, heads=heads)
             else:
                 item_seq, item_row0, item_npos, n_items = self._items(ctx, "attention.decode_items")
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,

@@ -292,7 +292,7 @@ def items_for(lib, starts, counts, group, per=None):
 
 def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1, seed=0,
                   boost=None, kernel="generic", waves=4, longest=None, key_ways=1,
-                  pair_items=True):
+                  pair_items=True, heads=0):
     """Fill a paged cache with random keys and values, run the kernel for the last
     `counts[b]` positions of each sequence, return (kernel output, plain output)."""
     torch.manual_seed(seed)
@@ -332,6 +332,7 @@ def run_attention(lib, dtype, nq, nkv, D, starts, counts, window=None, splits=1,
         lib.attention_decode_mfma(q.reshape(N, nq * D), cache.k, cache.v, pos, seq,
                                   cache.table_dev, out, nq, nkv, D, window=window,
                                   n_splits=splits, part_o=part_o, part_ml=part_ml, waves=waves,
+                                  heads=heads,
                                   longest=None if longest is None else torch.tensor(
                                       [longest], dtype=torch.int32, device=DEV))
     else:
@@ -417,6 +418,24 @@ def test_attention_decode_on_the_matrix_cores(lib, nq, nkv, D, splits, waves):
     close(out, expected, torch.bfloat16)
 
 
+@pytest.mark.parametrize("nq,nkv,D,splits", [(32, 8, 128, 1), (32, 8, 128, 4), (6, 2, 128, 2), (16, 1, 64, 3)])
+@pytest.mark.parametrize("waves,heads", [(16, 1), (16, 2), (8, 1), (8, 4), (4, 2)])
+def test_attention_decode_with_fewer_heads_a_block(lib, nq, nkv, D, splits, waves, heads):
+    """A block that takes fewer query heads of a group than it could (more, lighter blocks for
+    steps of few sequences): the same result, also where the group is no multiple of them."""
+    starts = [0, 15, 16, 63, 64, 300, 1029]
+    out, expected = run_attention(lib, torch.bfloat16, nq, nkv, D, starts=starts,
+                                  counts=[1] * len(starts), splits=splits, kernel="decode_mfma",
+                                  waves=waves, heads=heads, seed=11)
+    close(out, expected, torch.bfloat16)
+
+
+def test_attention_decode_refuses_heads_a_block_that_are_no_power_of_two(lib):
+    with pytest.raises(lib.KernelError, match="power of two"):
+        run_attention(lib, torch.bfloat16, 8, 2, 64, starts=[5], counts=[1], kernel="decode_mfma",
+                      waves=16, heads=3)
+
+
 @pytest.mark.parametrize("splits,waves", [(2, 4), (5, 4), (32, 4), (3, 16)])
 @pytest.mark.parametrize("longest", ["exact", "short", "long"])
 def test_attention_decode_slices_of_the_longest_sequences_share(lib, splits, waves, longest):
@@ -495,9 +514,12 @@ def test_attention_decode_from_the_projection(lib, nq, nkv, D, splits, waves, sl
             q = torch.full((N, nq * D), float("nan"), device=DEV, dtype=torch.bfloat16)
             lib.qk_norm_rope_store(qkv, qn, kn, eps, table, pos, seq, cache.table_dev, q,
                                    cache.k, cache.v, nq, nkv, D, write_cache=write)
+        # the fused run also with fewer heads a block than the block could take: every block of
+        # a group makes the position's key and value for itself, the first one stores them
+        heads = {"window": 1, "bare": 2}.get(options, 0) if fused else 0
         lib.attention_decode_mfma(q, cache.k, cache.v, pos, seq, cache.table_dev, out, nq, nkv, D,
                                   window=window, n_splits=splits, part_o=part_o, part_ml=part_ml,
-                                  waves=waves, longest=longest)
+                                  waves=waves, longest=longest, heads=heads)
         outs.append(out)
     separate, fused = outs
     assert torch.isnan(fused[3].float()).all() and torch.isnan(separate[3].float()).all()

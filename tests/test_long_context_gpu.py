@@ -151,10 +151,11 @@ def test_a_decode_batch_of_very_unequal_contexts(models, oracle, dtype):
                      f"{dtype} context {n} in an unequal batch")
     mixer = session.model.layers[0].mixer
     assert set(session._captured) == {(4, 4352)}
-    slices, waves = mixer.decode_launch(4, 4352)
+    slices, waves, heads = mixer.decode_launch(4, 4352)
     assert slices > 1, "this batch is meant to run the sliced launch shape"
     if mixer.matrix_cores:
-        assert waves == 16 and mixer.decode_launch(1, 300) == (1, 16)
+        # few blocks: a block takes one head of the group of two
+        assert waves == 16 and mixer.decode_launch(1, 300) == (1, 16, 1)
 
 
 @pytest.mark.parametrize("count,waves", [(72, 8), (136, 4)])
