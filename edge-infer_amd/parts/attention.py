@@ -125,6 +125,7 @@ class Attention:
         # case runs the generic kernel
         self.matrix_cores = (dtype == torch.bfloat16 and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
+        self._decode_launches = {}     # (sequences, context bound) -> decode_launch's answer
 
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self, key_ways: int = 1):
@@ -246,7 +247,11 @@ class Attention:
         out = ctx.buffer("attn.out", (n, spec.q_width))
         part_o = part_ml = None
         if ctx.decode:
-            splits, waves, heads = self.decode_launch(ctx.n_seqs, ctx.context_bound)
+            shape = (ctx.n_seqs, ctx.context_bound)
+            launch = self._decode_launches.get(shape)
+            if launch is None:          # (a step that is not replayed from a graph asks every layer)
+                launch = self._decode_launches[shape] = self.decode_launch(*shape)
+            splits, waves, heads = launch
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
                                     torch.float32)
