@@ -128,7 +128,14 @@ def _check(lib, status: int, what: str) -> None:
         raise KernelError(f"{what}: {message} (status {status})")
 
 
+# torch's own shortcut to the current stream's handle (no Stream object is made); a step of
+# few rows launches some 300 kernels and is bound by what each launch costs the host
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def _stream() -> int:
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
