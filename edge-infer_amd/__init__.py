@@ -53,6 +53,7 @@ def load_model(model_dir, dtype="bfloat16", device="cuda"):
 def random_model(cfg, seed, dtype="bfloat16", device="cuda", biases=False):
     """A model of configuration `cfg` with random weights drawn on the device (`biases`:
     with the optional bias of every projection and of the head)."""
+    from .config.registry import architecture_entry
     from .engine.model import DecoderModel, expected_parameters
     from .weights import random_parameters
 
@@ -61,7 +62,10 @@ def random_model(cfg, seed, dtype="bfloat16", device="cuda", biases=False):
     expected = expected_parameters(spec, cfg.checkpoint_name)
     skip = ("head.weight",) if spec.tie_word_embeddings else ()
     params = random_parameters(expected, seed, device=device, skip=skip, biases=biases)
-    model = DecoderModel(spec, params, dtype, device)
+    # the model class is the registry's, as for a model read from a folder
+    entry = architecture_entry(getattr(cfg, "architecture", spec.architecture))
+    factory = (entry.model_factory if entry is not None else None) or DecoderModel
+    model = factory(spec, params, dtype, device)
     model.config = cfg
     return model
 

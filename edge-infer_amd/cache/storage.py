@@ -5,8 +5,9 @@ it needs (`KVRequest`: keys and values per position, perhaps only a window of th
 `StateRequest`: a tensor of fixed size per sequence).  Entries with the same needs
 form a group with storage of its own:
 
-  key/value group   k, v: [entries, pages, kv_heads, 64, head_dim] in the storage
-                    type, a page pool, and per slot the list of its pages
+  key/value group   k: [entries, pages, kv_heads, 64, head_dim], v: the same with the
+                    group's value width, in the storage type; a page pool, and per
+                    slot the list of its pages
   state group       [entries, slots + 1, *shape] float32, zeroed when a slot is taken; the
                     last row is a spare that no sequence owns (padding of a fixed-size
                     batch points there, so kernels need no branch for it)
@@ -76,9 +77,10 @@ class SessionCache:
             pool = PagePool(self.n_pages)
             self.kv_pools.append(pool)
             self.kv_pages.append(SequencePages(pool, self.n_slots, window=request.window))
-            shape = (len(entries), self.n_pages, request.n_kv_heads, PAGE_TOKENS, request.head_dim)
-            self.kv_k.append(torch.empty(shape, dtype=dtype, device=device))
-            self.kv_v.append(torch.empty(shape, dtype=dtype, device=device))
+            shape = (len(entries), self.n_pages, request.n_kv_heads, PAGE_TOKENS)
+            value_dim = request.head_dim if request.value_dim is None else request.value_dim
+            self.kv_k.append(torch.empty(shape + (request.head_dim,), dtype=dtype, device=device))
+            self.kv_v.append(torch.empty(shape + (value_dim,), dtype=dtype, device=device))
         self._page_mirror: List[Dict[int, tuple]] = [{} for _ in self.kv_pages]
         self.states: List[torch.Tensor] = []
         self._state_copies: List[torch.Tensor] = []     # [slots, entries, *shape], see save_states

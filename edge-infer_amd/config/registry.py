@@ -17,7 +17,8 @@ from typing import Any, Callable, Dict, Mapping, Optional
 class Architecture:
     name: str
     config_class: Any                       # has from_dict(), model_spec(), checkpoint_name()
-    model_factory: Optional[Callable] = None  # (spec, dtype, device) -> model; None: DecoderModel
+    # (spec, params, dtype, device) -> model; None: engine.model.DecoderModel
+    model_factory: Optional[Callable] = None
     model_types: tuple = ()
 
 
@@ -37,6 +38,11 @@ def unregister_architecture(name: str) -> None:
     entry = _ARCHITECTURES.pop(name)
     for model_type in entry.model_types:
         _MODEL_TYPES.pop(model_type, None)
+
+
+def architecture_entry(name: str) -> Optional[Architecture]:
+    """The registered entry of an architecture's name, or None."""
+    return _ARCHITECTURES.get(name)
 
 
 def known_architectures():

@@ -31,8 +31,9 @@ __device__ __forceinline__ float bf16_hi(uint32_t u) { return __uint_as_float(u 
 // What a block needs to make its own queries, and the new key and value of its kv head, from
 // the fused projection (PREP): the work of the separate norm-rotate-store kernel, saved as a
 // launch per layer.  qkv: float32 partial sums [nsplit][rows, (nq + 2 nkv) * D], added in slice
-// order; per-head RMSNorm weights (or null); the rotation table [positions, D] (cosines, then
-// sines; or null); k_store / v_store: the cache pages to write the new key and value to (null:
+// order; per-head RMSNorm weights (or null); the rotation table [positions, rot_dim] (cosines,
+// then sines; or null; rot_dim <= D: pairs (i, i + rot_dim/2), the elements from rot_dim on
+// pass unrotated, as in rope_store.hip); k_store / v_store: the cache pages to write the new key and value to (null:
 // this run of the layer reads a cache that another run wrote, and has no key of its own).
 // Formulas and order as in rope_store.hip (runtime/include/execution/decoder.hpp:125-140).
 struct DecodePrep {
@@ -43,6 +44,7 @@ struct DecodePrep {
   const float* k_norm_w;
   float eps;
   const float* rope_table;
+  int rot_dim;
   bf16_t* k_store;
   bf16_t* v_store;
 };
@@ -98,33 +100,38 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     const int page_now = own_key
         ? page_table[static_cast<size_t>(seq) * table_width + pos / EI_PAGE] : -1;
     const bool active = lane < half;
-    const int i = active ? lane : 0;
+    // the lane's pair: elements (i, i2), rotated if it lies within the rotated width
+    const int rhalf = prep.rope_table != nullptr ? prep.rot_dim / 2 : half;
+    const int pair = active ? lane : 0;
+    const bool turned = pair < rhalf;
+    const int i = turned ? pair : pair + rhalf;
+    const int i2 = turned ? pair + rhalf : pair + half;
     for (int h = wave; h < heads_here + (own_key ? 2 : 0); h += W) {
       const int kind = h < heads_here ? 0 : (h == heads_here ? 1 : 2);   // query, key, value
       const int slot = kind == 0 ? h : GB + kind - 1;
       const int column = kind == 0 ? (head0 + h) * D
                                    : (kind == 1 ? (nq + g) * D : (nq + nkv + g) * D);
       const float* norm_w = kind == 0 ? prep.q_norm_w : (kind == 1 ? prep.k_norm_w : nullptr);
-      const bool rotate = kind != 2 && prep.rope_table != nullptr;
+      const bool rotate = kind != 2 && prep.rope_table != nullptr && turned;
       float wx = 1.f, wy = 1.f, cs = 1.f, sn = 0.f;
       if (norm_w != nullptr) {
         wx = norm_w[i];
-        wy = norm_w[i + half];
+        wy = norm_w[i2];
       }
       if (rotate) {
-        const float* trig = prep.rope_table + static_cast<size_t>(pos) * D;
-        cs = trig[i];
-        sn = trig[i + half];
+        const float* trig = prep.rope_table + static_cast<size_t>(pos) * (2 * rhalf);
+        cs = trig[pair];
+        sn = trig[pair + rhalf];
       }
       float x = 0.f, y = 0.f;
-      const float* p = src + column + i;
+      const float* p = src + column;
       for (int s0 = 0; s0 < prep.nsplit; s0 += 8) {       // slices in slice order, 8 per trip
         float xa[8], ya[8];
 #pragma unroll
         for (int u = 0; u < 8; ++u)
           if (s0 + u < prep.nsplit) {
-            xa[u] = p[(s0 + u) * prep.split_stride];
-            ya[u] = p[(s0 + u) * prep.split_stride + half];
+            xa[u] = p[(s0 + u) * prep.split_stride + i];
+            ya[u] = p[(s0 + u) * prep.split_stride + i2];
           }
 #pragma unroll
         for (int u = 0; u < 8; ++u)
@@ -150,12 +157,12 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
       if (active) {
         const bf16_t a16 = ei::from_f32<bf16_t>(a), b16 = ei::from_f32<bf16_t>(b);
         fin_lds[slot][i] = a16;
-        fin_lds[slot][i + half] = b16;
+        fin_lds[slot][i2] = b16;
         if (kind != 0 && hb == 0 && split == 0 && page_now >= 0) {
           bf16_t* dst = (kind == 1 ? prep.k_store : prep.v_store) +
                         ((static_cast<size_t>(page_now) * nkv + g) * EI_PAGE + pos % EI_PAGE) * D;
           dst[i] = a16;
-          dst[i + half] = b16;
+          dst[i2] = b16;
         }
       }
     }
@@ -939,7 +946,7 @@ extern "C" int ei_attention_prefill_mfma(const void* q, const void* k_pages, con
   // place is free, spread better (700 and 1,500 tokens: 65 against 90 us unpaired; 300, 900,
   // 2,000 and 4,000: 233 against 251), so their caller does not ask for pairs.
   const int pair =
-      pair_items && static_cast<long long>(n_items) * (G / HB) * nkv >= 2 * 256 ? 1 : 0;
+      pair_items && static_cast<long long>(n_items) * (G / HB) * nkv >= 2 * ei_compute_units() ? 1 : 0;
   const long long units = pair ? (n_items + 1) / 2 : n_items;
   const long long rests = units * (G / HB);
   long long blocks;
@@ -1077,15 +1084,19 @@ extern "C" int ei_attention_decode_mfma(const void* q, const void* k_pages, cons
 // (partial sums, added in slice order); the kernel norms and rotates its queries itself and,
 // with write_cache, also the position's key, and stores that key and the value in the pages
 // (so the separate norm-rotate-store kernel is not needed for these rows).  q_norm_w, k_norm_w
-// (float32 [D]) and rope_table (float32 [positions, D]) may each be null.
+// (float32 [D]) and rope_table (float32 [positions, rot_dim], rot_dim even and at most D) may
+// each be null.
 extern "C" int ei_attention_decode_mfma_fused(
     const float* qkv, int nsplit, long long split_stride, const float* q_norm_w,
-    const float* k_norm_w, float eps, const float* rope_table, int write_cache, void* k_pages,
+    const float* k_norm_w, float eps, const float* rope_table, int rot_dim, int write_cache,
+    void* k_pages,
     void* v_pages, const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table,
     int table_width, void* out, float* part_o, float* part_ml, int rows, int nq, int nkv, int D,
     int window, float scale, int n_splits, int waves, int heads, const int32_t* longest,
     hipStream_t stream) {
   EI_REQUIRE(qkv && nsplit >= 1 && split_stride >= 0, "attention_decode_fused: bad projection");
+  EI_REQUIRE(!rope_table || (rot_dim >= 2 && rot_dim % 2 == 0 && rot_dim <= D),
+             "attention_decode_fused: the rotated width must be even and at most head_dim");
   DecodePrep prep{};
   prep.qkv = qkv;
   prep.nsplit = nsplit;
@@ -1094,6 +1105,7 @@ extern "C" int ei_attention_decode_mfma_fused(
   prep.k_norm_w = k_norm_w;
   prep.eps = eps;
   prep.rope_table = rope_table;
+  prep.rot_dim = rope_table ? rot_dim : D;
   prep.k_store = write_cache ? static_cast<bf16_t*>(k_pages) : nullptr;
   prep.v_store = write_cache ? static_cast<bf16_t*>(v_pages) : nullptr;
   return decode_launch(nullptr, k_pages, v_pages, row_pos, row_seq, page_table, table_width, out,

@@ -135,6 +135,22 @@ static inline void ei_set_error(const char* message) {
 }
 extern "C" const char* ei_last_error() { return ei_error_text; }
 
+// Compute units of the current device, asked of the runtime once per device (256 on an
+// MI355X).  Launch plans that deal blocks out to the units take the count from here.
+static inline int ei_compute_units() {
+  static int known[64] = {0};
+  int device = 0;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return 256;
+  if (known[device] == 0) {
+    int count = 0;
+    if (hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess ||
+        count < 1)
+      count = 256;
+    known[device] = count;
+  }
+  return known[device];
+}
+
 #define EI_REQUIRE(cond, msg)       \
   do {                              \
     if (!(cond)) {                  \

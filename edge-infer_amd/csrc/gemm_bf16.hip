@@ -347,7 +347,6 @@ skinny_gemm_kernel(const bf16_t* __restrict__ W, const bf16_t* __restrict__ X,
 }
 
 constexpr int kTile = 256;                // K-tile of the kernel
-constexpr int kComputeUnits = 256;        // MI355X
 constexpr int kGroupRows = 64;            // rows of X one block takes
 constexpr int kMaxRows = 256;
 
@@ -359,6 +358,7 @@ constexpr int kMaxRows = 256;
 // on every strip group (more rows of X than one block takes).
 int tile_kernel_waves(int n_strips, int splits, int row_groups, double tiles_per_slice,
                       double* cost_out) {
+  const int kComputeUnits = ei_compute_units();
   int best = 8;
   double best_cost = 1e30;
   for (int waves = 8; waves >= 4; waves -= 2) {
@@ -393,6 +393,7 @@ extern "C" int ei_skinny_gemm_splits(int M, int N, int K, int max_splits) {
   const int k_tiles = (K + kTile - 1) / kTile;
   const int n_strips = (N + 15) / 16;
   if (max_splits <= 0 || max_splits > 16) max_splits = 16;
+  const int kComputeUnits = ei_compute_units();
   int best = 1;
   double best_cost = 1e30;
   for (int splits = 1; splits <= max_splits && splits <= k_tiles; ++splits) {

@@ -9,6 +9,7 @@ these functions: if a library cannot be built or loaded the call raises.
 from __future__ import annotations
 
 import ctypes
+import functools
 import os
 from ctypes import c_float, c_int, c_longlong, c_ulonglong, c_void_p
 from typing import Dict, Optional
@@ -55,7 +56,7 @@ _SIGNATURES = {
                                      c_int, c_int, c_float, c_int, c_int, c_int, c_void_p,
                                      c_void_p],
         "ei_attention_decode_mfma_fused": [c_void_p, c_int, c_longlong, c_void_p, c_void_p, c_float,
-                                           c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                                           c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                            c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_int,
                                            c_int, c_int, c_int, c_int, c_float, c_int, c_int,
                                            c_int, c_void_p, c_void_p],
@@ -131,6 +132,22 @@ def _check(lib, status: int, what: str) -> None:
 # torch's own shortcut to the current stream's handle (no Stream object is made); a step of
 # few rows launches some 300 kernels and is bound by what each launch costs the host
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+@functools.lru_cache(maxsize=None)
+def _compute_units(index: int) -> int:
+    return int(torch.cuda.get_device_properties(index).multi_processor_count)
+
+
+def compute_units(device=None) -> int:
+    """Compute units of a device (the current one by default): 256 on an MI355X.  The one
+    place on the Python side where launch plans take the chip's size from."""
+    if device is None:
+        index = torch.cuda.current_device()
+    else:
+        device = torch.device(device)
+        index = torch.cuda.current_device() if device.index is None else device.index
+    return _compute_units(index)
 
 
 def _stream() -> int:
@@ -240,9 +257,23 @@ def bias_rows(bias: torch.Tensor, out: torch.Tensor, accumulate: bool) -> None:
     _check(lib, status, "bias_rows")
 
 
+def _rotated_width(rope_table, head_dim: int, what: str) -> int:
+    """The width of a rotation table [positions, R]: R/2 cosines, then R/2 sines, for the
+    pairs (i, i + R/2) of a head's first R <= head_dim elements; the rest pass unrotated."""
+    if rope_table is None:
+        return head_dim
+    if rope_table.dim() != 2 or rope_table.shape[1] % 2 or not 2 <= rope_table.shape[1] <= head_dim:
+        raise KernelError(f"{what}: the rotation table must be [positions, R] with R even and at "
+                          f"most head_dim = {head_dim}, got {list(rope_table.shape)}")
+    return rope_table.shape[1]
+
+
 def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, eps, rope_table, row_pos, row_seq, page_table,
                        q_out, k_pages, v_pages, n_heads, n_kv_heads, head_dim,
                        write_cache=True) -> None:
+    """Per-head RMSNorm of queries and keys (weights or None), rotation by `rope_table`
+    (float32 [positions, R], R <= head_dim; or None), queries to `q_out`, keys and values to
+    their cache pages."""
     lib = library("rope_store")
     n = q_out.shape[0]
     width = (n_heads + 2 * n_kv_heads) * head_dim
@@ -251,11 +282,7 @@ def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, eps, rope_table, row_pos, row_se
         raise KernelError("qk_norm_rope_store: q_out has the wrong shape")
     if row_pos.numel() < n or row_seq.numel() < n:
         raise KernelError("qk_norm_rope_store: row metadata shorter than the rows")
-    max_pos = 0
-    if rope_table is not None:
-        if rope_table.dim() != 2 or rope_table.shape[1] != head_dim:
-            raise KernelError("qk_norm_rope_store: rope table must be [positions, head_dim]")
-        max_pos = rope_table.shape[0]
+    rot_dim = _rotated_width(rope_table, head_dim, "qk_norm_rope_store")
     if write_cache:
         expect = (n_kv_heads, PAGE_TOKENS, head_dim)
         if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
@@ -266,7 +293,7 @@ def qk_norm_rope_store(qkv, q_norm_w, k_norm_w, eps, rope_table, row_pos, row_se
         _gpu(qkv, "qkv"), _code(qkv, "qkv"), nsplit, stride,
         None if q_norm_w is None else _gpu(q_norm_w, "q_norm", torch.float32),
         None if k_norm_w is None else _gpu(k_norm_w, "k_norm", torch.float32), float(eps),
-        None if rope_table is None else _gpu(rope_table, "rope_table", torch.float32), max_pos,
+        None if rope_table is None else _gpu(rope_table, "rope_table", torch.float32), rot_dim,
         _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
         _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],
         _gpu(q_out, "q_out"), _gpu(k_pages, "k_pages") if write_cache else None,
@@ -345,13 +372,25 @@ def attention_prefill_mfma_positions(group: int, key_ways: int = 1) -> int:
 
 def attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items, row_pos,
                            page_table, out, n_heads, n_kv_heads, head_dim, window=None,
-                           scale=None, key_ways=1, pair_items=True) -> None:
+                           scale=None, key_ways=1, pair_items=True, largest_item=None) -> None:
     """bfloat16 prefill attention on the matrix cores; an item holds up to
     `attention_prefill_mfma_positions(group, key_ways)` positions of one sequence.
     pair_items: with enough items a block may take item i and then item n_items - 1 - i
-    (equal work a block where the items are those of one prompt, longest first)."""
+    (equal work a block where the items are those of one prompt, longest first).
+    largest_item: the most positions any item holds, from the host's copy of the list (the
+    kernel gives a block's waves fixed rows of an item and would leave the rows of a larger
+    one out); None: looked up from `item_npos` on the device, which waits for the device."""
     lib = library("attention_mfma")
     n = q.shape[0]
+    capacity = attention_prefill_mfma_positions(n_heads // max(1, n_kv_heads), key_ways)
+    if capacity == 0:
+        raise KernelError(f"attention_prefill: no form with key_ways = {key_ways} for groups of "
+                          f"{n_heads // max(1, n_kv_heads)} heads")
+    if largest_item is None:
+        largest_item = int(item_npos[:n_items].max().item())
+    if not 0 <= int(largest_item) <= capacity:
+        raise KernelError(f"attention_prefill: an item of {largest_item} positions; a block "
+                          f"takes at most {capacity} with key_ways = {key_ways}")
     if tuple(q.shape) != (n, n_heads * head_dim) or tuple(out.shape) != tuple(q.shape):
         raise KernelError("attention_prefill: q and out must be [rows, heads * head_dim]")
     expect = (n_kv_heads, PAGE_TOKENS, head_dim)
@@ -376,7 +415,7 @@ class DecodeProjection:
     """What `attention_decode_mfma` needs to make queries, key and value itself: the fused
     projection as float32 partial sums [slices, rows, (heads + 2 kv heads) * head_dim], the
     per-head RMSNorm weights (float32 [head_dim], or None), their eps, the rotation table
-    (float32 [positions, head_dim], or None), and whether the position's key and value are
+    (float32 [positions, R] with R <= head_dim, or None), and whether the position's key and value are
     stored in the pages."""
 
     def __init__(self, qkv, q_norm_w, k_norm_w, eps, rope_table, write_cache):
@@ -410,9 +449,7 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
             weight = getattr(q, name)
             if weight is not None and weight.numel() != head_dim:
                 raise KernelError(f"attention_decode: {name} must have {head_dim} elements")
-        if q.rope_table is not None and (q.rope_table.dim() != 2
-                                         or q.rope_table.shape[1] != head_dim):
-            raise KernelError("attention_decode: rope table must be [positions, head_dim]")
+        rot_dim = _rotated_width(q.rope_table, head_dim, "attention_decode")
     expect = (n_kv_heads, PAGE_TOKENS, head_dim)
     if tuple(k_pages.shape[1:]) != expect or tuple(v_pages.shape) != tuple(k_pages.shape):
         raise KernelError(f"attention_decode: pages must be [*, {expect}]")
@@ -430,7 +467,7 @@ def attention_decode_mfma(q, k_pages, v_pages, row_pos, row_seq, page_table, out
         status = lib.ei_attention_decode_mfma_fused(
             _gpu(q.qkv, "qkv", torch.float32), q.qkv.shape[0], n * width,
             opt(q.q_norm_w, "q_norm"), opt(q.k_norm_w, "k_norm"), float(q.eps),
-            opt(q.rope_table, "rope_table"), int(bool(q.write_cache)),
+            opt(q.rope_table, "rope_table"), rot_dim, int(bool(q.write_cache)),
             _gpu(k_pages, "k_pages", torch.bfloat16), _gpu(v_pages, "v_pages", torch.bfloat16),
             _gpu(row_pos, "row_pos", torch.int32), _gpu(row_seq, "row_seq", torch.int32),
             _gpu(page_table, "page_table", torch.int32), page_table.shape[-1],

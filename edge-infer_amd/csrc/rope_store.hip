@@ -10,6 +10,11 @@
 // runtime/include/execution/decoder.hpp:125-140; rotate-half pairs (i, i + d/2),
 // x' = x cos - y sin, y' = x sin + y cos, operators/src/cuda/execution.cu:79-122;
 // keys stored after norm and rotation, values raw, decoder.hpp:137-140.
+//
+// The rotation may cover only the first R <= D elements of a head (R = the table's width):
+// pairs (i, i + R/2) for i < R/2, elements R..D-1 pass unrotated.  A lane's pair j of D/2 is
+// then elements (j, j + R/2) below R/2 and (j + R/2, j + D/2) from there on, the latter with
+// the identity as its rotation; with R = D this is the pair (j, j + D/2) throughout.
 #include "common.h"
 
 namespace {
@@ -20,11 +25,11 @@ template <typename TI, typename TO>
 __global__ void qk_norm_rope_store_kernel(
     const TI* __restrict__ qkv, int nsplit, size_t split_stride,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
-    const float* __restrict__ rope_table,  // [max_pos, D]: cos[D/2] then sin[D/2]; null: none
+    const float* __restrict__ rope_table,  // [max_pos, R]: cos[R/2] then sin[R/2]; null: none
     const int32_t* __restrict__ row_pos, const int32_t* __restrict__ row_seq,
     const int32_t* __restrict__ page_table, int table_width,
     TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
-    int N, int nq, int nkv, int D, int write_cache) {
+    int N, int nq, int nkv, int D, int R, int write_cache) {
   const int heads = nq + 2 * nkv;
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / EI_WAVE;
   const int lane = threadIdx.x % EI_WAVE;
@@ -35,7 +40,7 @@ __global__ void qk_norm_rope_store_kernel(
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
   if (!is_q && !write_cache) return;
   const int pos = row_pos[row];
-  const int half = D / 2;
+  const int half = D / 2, rhalf = R / 2;
   const size_t width = static_cast<size_t>(nq + 2 * nkv) * D;
   const TI* src = qkv + static_cast<size_t>(row) * width + static_cast<size_t>(head) * D;
 
@@ -43,10 +48,12 @@ __global__ void qk_norm_rope_store_kernel(
   float sum = 0.f;
 #pragma unroll
   for (int j = 0; j < kMaxPairsPerLane; ++j) {
-    const int i = lane + j * EI_WAVE;
+    const int pair = lane + j * EI_WAVE;
     x[j] = 0.f;
     y[j] = 0.f;
-    if (i < half) {
+    if (pair < half) {
+      const int i = pair < rhalf ? pair : pair + rhalf;          // the pair's first element
+      const int i2 = pair < rhalf ? pair + rhalf : pair + half;  // and its second
       // slices are added in slice order, four loads per trip to memory
       for (int s0 = 0; s0 < nsplit; s0 += 4) {
         TI a[4], b[4];
@@ -54,7 +61,7 @@ __global__ void qk_norm_rope_store_kernel(
         for (int u = 0; u < 4; ++u)
           if (s0 + u < nsplit) {
             a[u] = src[(s0 + u) * split_stride + i];
-            b[u] = src[(s0 + u) * split_stride + i + half];
+            b[u] = src[(s0 + u) * split_stride + i2];
           }
 #pragma unroll
         for (int u = 0; u < 4; ++u)
@@ -85,32 +92,34 @@ __global__ void qk_norm_rope_store_kernel(
     inv = rsqrtf(sum / static_cast<float>(D) + eps);
   }
   const bool rotate = rope_table != nullptr && (is_q || is_k);
-  const float* trig = rotate ? rope_table + static_cast<size_t>(pos) * D : nullptr;
+  const float* trig = rotate ? rope_table + static_cast<size_t>(pos) * R : nullptr;
 #pragma unroll
   for (int j = 0; j < kMaxPairsPerLane; ++j) {
-    const int i = lane + j * EI_WAVE;
-    if (i < half) {
+    const int pair = lane + j * EI_WAVE;
+    if (pair < half) {
+      const int i = pair < rhalf ? pair : pair + rhalf;
+      const int i2 = pair < rhalf ? pair + rhalf : pair + half;
       float a = x[j], b = y[j];
       if (norm_w) {
         a = (a * inv) * norm_w[i];
-        b = (b * inv) * norm_w[i + half];
+        b = (b * inv) * norm_w[i2];
       }
-      if (rotate) {
-        const float c = trig[i], s = trig[i + half];
+      if (rotate && pair < rhalf) {
+        const float c = trig[pair], s = trig[pair + rhalf];
         const float ra = a * c - b * s;
         const float rb = a * s + b * c;
         a = ra;
         b = rb;
       }
       dst[i] = ei::from_f32<TO>(a);
-      dst[i + half] = ei::from_f32<TO>(b);
+      dst[i2] = ei::from_f32<TO>(b);
     }
   }
 }
 
-// The same for head sizes that are a multiple of 8: G lanes (a power of two) share a head,
-// each lane takes 4 neighbouring pairs with one 8- or 16-byte access per half, so a wave
-// covers 64 / G heads.
+// The same for head sizes (and rotated widths) that are a multiple of 8: G lanes (a power of
+// two) share a head, each lane takes 4 neighbouring pairs with one 8- or 16-byte access per
+// half, so a wave covers 64 / G heads.
 template <typename TI, typename TO, int G>
 __global__ void qk_norm_rope_store_vec_kernel(
     const TI* __restrict__ qkv, int nsplit, size_t split_stride,
@@ -118,7 +127,7 @@ __global__ void qk_norm_rope_store_vec_kernel(
     const float* __restrict__ rope_table, const int32_t* __restrict__ row_pos,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
     TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
-    int N, int nq, int nkv, int D, int write_cache) {
+    int N, int nq, int nkv, int D, int R, int write_cache) {
   using ei::Vec4;
   const int heads = nq + 2 * nkv;
   const long long item = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) / G;
@@ -130,11 +139,14 @@ __global__ void qk_norm_rope_store_vec_kernel(
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
   if (!is_q && !write_cache) return;
   const int pos = row_pos[row];
-  const int half = D / 2;
-  const int i0 = sub * 4;
-  const bool active = i0 < half;
+  const int half = D / 2, rhalf = R / 2;
+  const int pair0 = sub * 4;                                   // the lane's first pair
+  const bool active = pair0 < half;
+  const bool turned = pair0 < rhalf;                           // its four pairs are rotated ones
+  const int i0 = turned ? pair0 : pair0 + rhalf;               // their first elements
+  const int i2 = turned ? pair0 + rhalf : pair0 + half;        // and their second ones
   const size_t width = static_cast<size_t>(heads) * D;
-  const TI* src = qkv + static_cast<size_t>(row) * width + static_cast<size_t>(head) * D + i0;
+  const TI* src = qkv + static_cast<size_t>(row) * width + static_cast<size_t>(head) * D;
 
   TO* dst;
   bool stored = true;
@@ -159,8 +171,8 @@ __global__ void qk_norm_rope_store_vec_kernel(
 #pragma unroll
       for (int u = 0; u < 4; ++u)
         if (s0 + u < nsplit) {
-          Vec4<TI>::load(src + (s0 + u) * split_stride, a[u]);
-          Vec4<TI>::load(src + (s0 + u) * split_stride + half, b[u]);
+          Vec4<TI>::load(src + (s0 + u) * split_stride + i0, a[u]);
+          Vec4<TI>::load(src + (s0 + u) * split_stride + i2, b[u]);
         }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
@@ -174,12 +186,12 @@ __global__ void qk_norm_rope_store_vec_kernel(
     }
     if (norm_w) {
       Vec4<float>::load(norm_w + i0, wx);
-      Vec4<float>::load(norm_w + i0 + half, wy);
+      Vec4<float>::load(norm_w + i2, wy);
     }
-    if (rotate) {
-      const float* trig = rope_table + static_cast<size_t>(pos) * D + i0;
+    if (rotate && turned) {
+      const float* trig = rope_table + static_cast<size_t>(pos) * R + pair0;
       Vec4<float>::load(trig, cs);
-      Vec4<float>::load(trig + half, sn);
+      Vec4<float>::load(trig + rhalf, sn);
     }
   }
   float inv = 1.f;
@@ -200,7 +212,7 @@ __global__ void qk_norm_rope_store_vec_kernel(
       a = (a * inv) * wx[i];
       b = (b * inv) * wy[i];
     }
-    if (rotate) {
+    if (rotate) {                      // (the identity for pairs beyond the rotated width)
       const float ra = a * cs[i] - b * sn[i];
       const float rb = a * sn[i] + b * cs[i];
       a = ra;
@@ -210,7 +222,7 @@ __global__ void qk_norm_rope_store_vec_kernel(
     oy[i] = b;
   }
   Vec4<TO>::store(dst + i0, ox);
-  Vec4<TO>::store(dst + i0 + half, oy);
+  Vec4<TO>::store(dst + i2, oy);
 }
 
 }  // namespace
@@ -220,7 +232,7 @@ __global__ void qk_norm_rope_store_vec_kernel(
 // page_table: int32 [n_seqs, table_width], logical page -> physical page.
 extern "C" int ei_qk_norm_rope_store(
     const void* qkv, int in_dtype, int nsplit, long long split_stride, const float* q_norm_w,
-    const float* k_norm_w, float eps, const float* rope_table, int max_pos,
+    const float* k_norm_w, float eps, const float* rope_table, int rot_dim,
     const int32_t* row_pos, const int32_t* row_seq, const int32_t* page_table, int table_width,
     void* q_out, void* k_pages, void* v_pages, int out_dtype, int N, int nq, int nkv, int D,
     int write_cache, hipStream_t stream) {
@@ -231,7 +243,10 @@ extern "C" int ei_qk_norm_rope_store(
   EI_REQUIRE(!write_cache || (k_pages && v_pages && page_table && table_width > 0),
              "qk_norm_rope_store: cache pointers missing");
   EI_REQUIRE(nsplit >= 1, "qk_norm_rope_store: nsplit must be at least 1");
-  (void)max_pos;
+  // the rotated width R: the table's row length, even, at most the head size (D without a table)
+  const int R = rope_table ? rot_dim : D;
+  EI_REQUIRE(R >= 2 && R % 2 == 0 && R <= D,
+             "qk_norm_rope_store: the rotated width must be even and at most head_dim");
   const int heads = nq + 2 * nkv;
   const int threads = 256;
   const size_t ss = static_cast<size_t>(split_stride);
@@ -240,7 +255,7 @@ extern "C" int ei_qk_norm_rope_store(
                         reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(v_pages) |
                         reinterpret_cast<uintptr_t>(q_norm_w) | reinterpret_cast<uintptr_t>(k_norm_w) |
                         reinterpret_cast<uintptr_t>(rope_table)) % 16 == 0;
-  if (D % 8 == 0 && ss % 4 == 0 && aligned) {
+  if (D % 8 == 0 && R % 8 == 0 && ss % 4 == 0 && aligned) {
     int G = 1;
     while (G * 8 < D) G *= 2;
     const long long items = static_cast<long long>(N) * heads;
@@ -250,7 +265,7 @@ extern "C" int ei_qk_norm_rope_store(
   qk_norm_rope_store_vec_kernel<TI, TO, GG><<<static_cast<unsigned>(blocks), threads, 0, stream>>>( \
       static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, rope_table, row_pos,      \
       row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),       \
-      static_cast<TO*>(v_pages), N, nq, nkv, D, write_cache)
+      static_cast<TO*>(v_pages), N, nq, nkv, D, R, write_cache)
 #define EI_ROPE_VEC_G(TI, TO)                                                                     \
   do {                                                                                            \
     if (G <= 2) EI_ROPE_VEC(TI, TO, 2);                                                           \
@@ -280,7 +295,7 @@ extern "C" int ei_qk_norm_rope_store(
   qk_norm_rope_store_kernel<TI, TO><<<static_cast<unsigned>(blocks), threads, 0, stream>>>(      \
       static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, rope_table, row_pos,     \
       row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),      \
-      static_cast<TO*>(v_pages), N, nq, nkv, D, write_cache)
+      static_cast<TO*>(v_pages), N, nq, nkv, D, R, write_cache)
   if (in_dtype == EI_F32 && out_dtype == EI_F32)
     EI_ROPE_LAUNCH(float, float);
   else if (in_dtype == EI_F32 && out_dtype == EI_BF16)

@@ -244,7 +244,7 @@ extern "C" int ei_bias_rows(const float* bias, float* out, long long rows, int w
   const size_t n = static_cast<size_t>(rows) * width;
   const int threads = 256;
   size_t blocks = (n + threads - 1) / threads;
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
   bias_rows_kernel<<<static_cast<unsigned>(blocks), threads, 0, stream>>>(bias, out, n, width,
                                                                          accumulate);
   EI_LAUNCH_CHECK();
@@ -255,7 +255,7 @@ extern "C" int ei_sum_slices(const float* in, int nsplit, long long stride, floa
   EI_REQUIRE(in && out && nsplit >= 1 && n > 0 && stride >= n, "sum_slices: bad arguments");
   const int threads = 256;
   long long blocks = (n + threads - 1) / threads;
-  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks > ei_compute_units() * 16) blocks = ei_compute_units() * 16;
   sum_slices_kernel<<<static_cast<unsigned>(blocks), threads, 0, stream>>>(
       in, nsplit, static_cast<size_t>(stride), out, static_cast<size_t>(n));
   EI_LAUNCH_CHECK();
@@ -358,7 +358,7 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
   if (I % 8 == 0 && ss % 8 == 0 && strip % 8 == 0) {
     const size_t octets = total / 8;
     size_t vblocks = (octets + threads - 1) / threads;
-    if (vblocks > 256 * 32) vblocks = 256 * 32;
+    if (vblocks > ei_compute_units() * 32) vblocks = ei_compute_units() * 32;
     if (in_dtype == EI_F32 && out_dtype == EI_F32)
       swiglu_vec_kernel<float, float><<<vblocks, threads, 0, stream>>>(
           static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, octets, strip);
@@ -373,7 +373,7 @@ extern "C" int ei_swiglu(const void* gate_up, int in_dtype, int nsplit, long lon
     EI_LAUNCH_CHECK();
   }
   size_t blocks = (total + threads - 1) / threads;
-  if (blocks > 256 * 32) blocks = 256 * 32;
+  if (blocks > ei_compute_units() * 32) blocks = ei_compute_units() * 32;
   if (in_dtype == EI_F32 && out_dtype == EI_F32)
     swiglu_kernel<float, float><<<blocks, threads, 0, stream>>>(
         static_cast<const float*>(gate_up), nsplit, ss, static_cast<float*>(out), I, total, strip);

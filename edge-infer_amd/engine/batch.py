@@ -154,6 +154,7 @@ class DeviceMeta:
         self._device_buffer: Optional[torch.Tensor] = None
         self._host_buffer: Optional[torch.Tensor] = None
         self._views: Dict[str, torch.Tensor] = {}
+        self._host_sections: Dict[str, np.ndarray] = {}
         self._table_widths: List[int] = []
         self.n_seqs = 0
         self.n_want = 0
@@ -203,6 +204,7 @@ class DeviceMeta:
             if self._copied is None:
                 self._copied = torch.cuda.Event()
             self._copied.record()
+        self._host_sections = dict(sections)
         self._table_widths = [table.shape[1] for table in page_tables]
         self.n_seqs = plan.n_seqs
         self.n_want = int(plan.want_rows.size)
@@ -215,6 +217,14 @@ class DeviceMeta:
         except KeyError:
             raise KeyError(f"the step's metadata holds no section '{name}'; "
                            f"it holds {sorted(self._views)}") from None
+
+    def host_section(self, name: str) -> np.ndarray:
+        """The host's copy of a section as the last upload held it (flat int32): what a part
+        planned, for checks that must not wait for the device."""
+        try:
+            return self._host_sections[name]
+        except KeyError:
+            raise KeyError(f"the step's metadata holds no section '{name}'") from None
 
     longest = property(lambda self: self.section("longest"))
     tokens = property(lambda self: self.section("tokens"))

@@ -8,6 +8,19 @@ rows of a `StepContext` and returns float32 logits at the wanted rows.
 Order of operations: runtime/include/execution/decoder.hpp:109-171 and
 runtime/src/qwen3.cpp:293-299 of the reference (embedding, blocks, final norm,
 head); the head is applied to the wanted rows only.
+
+The skeleton around the layers is four methods, each of which an architecture may
+replace in a subclass that it registers as its `model_factory`, keeping the rest:
+
+  embed_rows(ctx) -> residual                 float32 [rows, hidden] in the buffer "residual"
+  run_layers(ctx, residual) -> pending        the layers in schedule order; the last delta,
+                                              not yet added to the residual
+  final_hidden(ctx, residual, pending) -> h   [wanted rows, hidden] in the storage type
+  logits(ctx, h) -> float32 [wanted rows, vocab]
+
+(a scaled embedding overrides `embed`, a cap on the logits `logits`, a model without a
+final norm `final_hidden`).  A subclass whose methods launch anything that a HIP graph
+cannot hold says so with `seams_capture_safe = False`; decode then runs eagerly.
 """
 from __future__ import annotations
 
@@ -190,11 +203,15 @@ class DecoderModel:
         for part in self._planners():
             plan.add_sections(part.plan_step(plan))
 
+    seams_capture_safe = True     # embed / final_hidden / logits launch only capturable work
+
     def capture_safe(self) -> bool:
         """Whether a decode step may be captured in a HIP graph: the final norm, the head,
         every block and every part of a block must say so with `capture_safe` (it launches
         nothing but capturable kernels and allocates nothing per step; a part that does not
-        say so is taken to be unsafe)."""
+        say so is taken to be unsafe), and so must the model's own methods around them."""
+        if not self.seams_capture_safe:
+            return False
         parts = [self.final_norm, self.head]
         for layer in self.layers:
             parts += [layer, *members_of(layer)]
@@ -243,16 +260,36 @@ class DecoderModel:
         return logits
 
     def _forward(self, ctx) -> torch.Tensor:
-        spec = self.spec
-        meta = ctx.meta
-        residual = ctx.buffer("residual", (ctx.n_rows, spec.hidden_size), torch.float32)
-        lib.embed_gather(meta.tokens, self.embed, residual)
-        pending = None
-        for entry in spec.schedule:
-            pending = self.layers[entry.layer].forward(ctx, residual, pending, entry)
-        if meta.n_want == 0:
-            return torch.empty((0, spec.vocab_size), dtype=torch.float32, device=self.device)
-        hidden = self.final_norm.add_norm(ctx, residual, pending, "final.h", rows=meta.want_rows,
-                                          write_residual=False)
+        residual = self.embed_rows(ctx)
+        pending = self.run_layers(ctx, residual)
+        if ctx.meta.n_want == 0:
+            return torch.empty((0, self.spec.vocab_size), dtype=torch.float32,
+                               device=self.device)
+        hidden = self.final_hidden(ctx, residual, pending)
         ctx.release(pending)
+        return self.logits(ctx, hidden)
+
+    # -- the skeleton: what a subclass may replace -------------------------------
+    def embed_rows(self, ctx) -> torch.Tensor:
+        """The rows of the embedding table that the step's tokens name, as the float32
+        residual stream [rows, hidden]."""
+        residual = ctx.buffer("residual", (ctx.n_rows, self.spec.hidden_size), torch.float32)
+        lib.embed_gather(ctx.meta.tokens, self.embed, residual)
+        return residual
+
+    def run_layers(self, ctx, residual):
+        """The layers in the order of the schedule.  Returns the last delta, which is not
+        added to the residual yet (the norm that follows adds it while it reads the row)."""
+        pending = None
+        for entry in self.spec.schedule:
+            pending = self.layers[entry.layer].forward(ctx, residual, pending, entry)
+        return pending
+
+    def final_hidden(self, ctx, residual, pending) -> torch.Tensor:
+        """The normalised rows that the head reads: only the wanted ones."""
+        return self.final_norm.add_norm(ctx, residual, pending, "final.h",
+                                        rows=ctx.meta.want_rows, write_residual=False)
+
+    def logits(self, ctx, hidden) -> torch.Tensor:
+        """float32 [wanted rows, vocab] in the buffer "logits"."""
         return self.head.forward_f32(ctx, hidden, "logits")

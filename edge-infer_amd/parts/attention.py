@@ -27,12 +27,13 @@ from .linear import Linear
 FUSED_DECODE = os.environ.get("EDGE_INFER_FUSED_DECODE", "1") != "0"
 
 
-# What the matrix-core decode kernel costs, measured on an MI355X (head size 128): a wave
-# walks a tile of 16 keys in 1.9 us; merging slices costs 4.5 us and 0.1 us a slice.
-TILE_US, MERGE_US, MERGE_SLICE_US = 1.9, 4.5, 0.1
-COMPUTE_UNITS = 256
-WAVE_SLOTS = COMPUTE_UNITS * 16     # waves the chip holds at once: compute units x waves a unit
+# What the matrix-core decode kernel costs, measured on an MI355X: a wave walks a tile of 16
+# keys of head size 128 in 1.9 us (other head sizes in proportion: a tile's bytes are what it
+# waits for); merging slices costs 4.5 us and 0.1 us a slice.
+TILE_US_128, MERGE_US, MERGE_SLICE_US = 1.9, 4.5, 0.1
+WAVES_A_UNIT = 16       # waves of this kernel that a compute unit holds at once
 MAX_SLICES = 32
+MAX_LAUNCH_PLANS = 512  # decode launch shapes a part remembers
 
 
 @functools.lru_cache(maxsize=512)
@@ -125,7 +126,8 @@ class Attention:
         # case runs the generic kernel
         self.matrix_cores = (dtype == torch.bfloat16 and
                             lib.attention_decode_mfma_supported(spec.head_dim, self.group))
-        self._decode_launches = {}     # (sequences, context bound) -> decode_launch's answer
+        self.compute_units = lib.compute_units(device)     # the chip's size, for launch plans
+        self._decode_launches = {}     # (sequences, pages of context) -> decode_launch's answer
 
     # the number of positions of one sequence that a prefill work item covers
     def positions_per_item(self, key_ways: int = 1):
@@ -146,7 +148,7 @@ class Attention:
         heads = lib.attention_prefill_mfma_heads(self.group)
         items = sum((count + size - 1) // size for count in counts)
         blocks = items * (self.group // heads) * self.spec.n_kv_heads
-        return 2 if blocks < 512 else 1
+        return 2 if blocks < 2 * self.compute_units else 1
 
     @property
     def plan_key(self):
@@ -183,29 +185,35 @@ class Attention:
     def decode_launch(self, n_seqs: int, context: int):
         """(slices of the key range, waves a block, query heads of a group a block takes) of
         a decode step over `n_seqs` sequences of up to `context` tokens.  A slice is the same
-        number of pages for every sequence.
+        number of pages for every sequence.  A layer with a window reads at most the window's
+        keys (and the rest of the page they begin in), so its slices are sized for those.
 
-        Matrix-core kernel, up to 256 (sequence, kv head) pairs: blocks of 16 waves, a tile
-        of 16 keys per wave at a time, and as many slices as shorten a wave's walk by more
-        than the merge kernel costs, while all blocks still fit the chip at once; if they
-        then leave compute units empty, a block takes fewer heads (2 or 1 instead of 4), as
-        long as every block still has a unit of its own: the keys are fetched once more per
-        block, from the L2, and each block has less to do per tile.  Up to 512 pairs: blocks
-        of 8 waves, no slices.  More pairs, and the generic kernel: blocks of 4 waves and
-        enough slices to put about two blocks on each of the 256 compute units, never more
-        than there are pages."""
+        Matrix-core kernel, up to as many (sequence, kv head) pairs as the chip has compute
+        units: blocks of 16 waves, a tile of 16 keys per wave at a time, and as many slices as
+        shorten a wave's walk by more than the merge kernel costs, while all blocks still fit
+        the chip at once; if they then leave compute units empty, a block takes fewer heads (2
+        or 1 instead of 4), as long as every block still has a unit of its own: the keys are
+        fetched once more per block, from the L2, and each block has less to do per tile.  Up
+        to twice as many pairs: blocks of 8 waves, no slices.  More pairs, and the generic
+        kernel: blocks of 4 waves and enough slices to put about two blocks on each compute
+        unit, never more than there are pages."""
+        if self.spec.window is not None:
+            context = min(context, self.spec.window + PAGE_TOKENS - 1)
         pages = max(1, (context + PAGE_TOKENS - 1) // PAGE_TOKENS)
         n_kv_heads = self.spec.n_kv_heads
+        units = self.compute_units
         if self.matrix_cores:
             # a block of 16 waves takes at most 4 query heads of a group: larger groups have
             # several blocks per pair
             pairs = n_seqs * n_kv_heads * ((self.group + 3) // 4)
-            if pairs <= 256:
+            if pairs <= units:
+                tile_us = TILE_US_128 * self.spec.head_dim / 128
                 tiles = (context + 15) // 16
-                best, best_cost = 1, TILE_US * ((tiles + 15) // 16)
+                best, best_cost = 1, tile_us * ((tiles + 15) // 16)
                 slices = 2
-                while slices <= min(pages, MAX_SLICES) and pairs * 16 * slices <= WAVE_SLOTS:
-                    cost = (TILE_US * ((tiles + 16 * slices - 1) // (16 * slices)) + MERGE_US
+                while (slices <= min(pages, MAX_SLICES)
+                       and pairs * 16 * slices <= units * WAVES_A_UNIT):
+                    cost = (tile_us * ((tiles + 16 * slices - 1) // (16 * slices)) + MERGE_US
                             + MERGE_SLICE_US * slices)
                     if cost < best_cost:
                         best, best_cost = slices, cost
@@ -213,18 +221,32 @@ class Attention:
                 heads = min(4, 1 << (self.group.bit_length() - 1))
                 while heads > 1:
                     blocks = n_seqs * n_kv_heads * best * -(-self.group // (heads // 2))
-                    if blocks > COMPUTE_UNITS:
+                    if blocks > units:
                         break
                     heads //= 2
                 return best, 16, heads
-            # up to 512 pairs of at most 8 heads: blocks of 8 waves fill the chip's wave slots
-            # once without slices (measured 1 to 3 % ahead of 4 waves at 32 to 64 sequences)
+            # up to twice as many pairs of at most 8 heads: blocks of 8 waves fill the chip's
+            # wave slots once without slices (measured 1 to 3 % ahead of 4 waves at 32 to 64
+            # sequences)
             pairs = n_seqs * n_kv_heads * ((self.group + 7) // 8)
-            if pairs <= 512:
+            if pairs <= 2 * units:
                 return 1, 8, 0
         blocks = n_seqs * n_kv_heads
-        wanted = (512 + blocks - 1) // blocks
+        wanted = (2 * units + blocks - 1) // blocks
         return max(1, min(wanted, pages, MAX_SLICES)), 4, 0
+
+    def _decode_launch_for(self, n_seqs: int, context: int):
+        """`decode_launch`, remembered per (sequences, pages of context): a step that is not
+        replayed from a graph asks in every layer and for every length, and the answer changes
+        with the pages at most."""
+        pages = (context + PAGE_TOKENS - 1) // PAGE_TOKENS
+        launch = self._decode_launches.get((n_seqs, pages))
+        if launch is None:
+            if len(self._decode_launches) >= MAX_LAUNCH_PLANS:
+                self._decode_launches.clear()
+            launch = self._decode_launches[(n_seqs, pages)] = \
+                self.decode_launch(n_seqs, pages * PAGE_TOKENS)
+        return launch
 
     def forward(self, ctx, x, entry):
         spec = self.spec
@@ -247,11 +269,7 @@ class Attention:
         out = ctx.buffer("attn.out", (n, spec.q_width))
         part_o = part_ml = None
         if ctx.decode:
-            shape = (ctx.n_seqs, ctx.context_bound)
-            launch = self._decode_launches.get(shape)
-            if launch is None:          # (a step that is not replayed from a graph asks every layer)
-                launch = self._decode_launches[shape] = self.decode_launch(*shape)
-            splits, waves, heads = launch
+            splits, waves, heads = self._decode_launch_for(ctx.n_seqs, ctx.context_bound)
             if splits > 1:
                 part_o = ctx.buffer("attn.part_o", (n * spec.n_heads * splits * spec.head_dim,),
                                     torch.float32)
@@ -271,14 +289,20 @@ class Attention:
                               scale=self.scale, n_splits=splits, part_o=part_o, part_ml=part_ml)
         else:
             key_ways = self.prefill_key_ways([seq.count for seq in ctx.sequences])
-            item_seq, item_row0, item_npos, n_items = self._items(
-                ctx, self._items_section(key_ways))
+            section = self._items_section(key_ways)
+            item_seq, item_row0, item_npos, n_items = self._items(ctx, section)
             if self.matrix_cores:
+                # the largest item of the list as the host planned it: the kernel's blocks
+                # hold a fixed number of rows and are told how many that must cover
+                largest = ctx.notes.get(section)
+                if largest is None:
+                    largest = ctx.notes[section] = int(ctx.meta.host_section(section)[2 * n_items:].max())
                 lib.attention_prefill_mfma(q, k_pages, v_pages, item_seq, item_row0, item_npos,
                                            n_items, meta.row_pos, page_table, out, spec.n_heads,
                                            spec.n_kv_heads, spec.head_dim, window=spec.window,
                                            scale=self.scale, key_ways=key_ways,
-                                           pair_items=len({(seq.start, seq.count) for seq in ctx.sequences}) == 1)
+                                           pair_items=len({(seq.start, seq.count) for seq in ctx.sequences}) == 1,
+                                           largest_item=largest)
             else:
                 lib.attention(q, k_pages, v_pages, item_seq, item_row0, item_npos, n_items,
                               meta.row_pos, meta.row_seq, page_table, out, spec.n_heads,

@@ -24,10 +24,13 @@ import torch
 
 @dataclass(frozen=True)
 class KVRequest:
-    """Keys and values for every position (or the last `window`) of a sequence."""
+    """Keys and values for every position (or the last `window`) of a sequence: pages
+    [kv_heads, 64, head_dim] of keys and [kv_heads, 64, value_dim] of values (`value_dim`
+    None: as wide as the keys)."""
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+    value_dim: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -239,6 +242,7 @@ class StepContext:
         self.context_bound = max_context if context_bound is None else context_bound
         self.fixed_shape = fixed_shape
         self.sequences = ()             # engine.batch.SeqStep of every live sequence (host)
+        self.notes = {}                 # what parts work out once a step and share between layers
 
     def buffer(self, name, shape, dtype=None):
         return self.workspace.get(name, shape, self.dtype if dtype is None else dtype)

@@ -27,6 +27,12 @@ TINY_B = dict(vocab_size=381, hidden_size=96, num_hidden_layers=3, num_attention
               num_key_value_heads=1, head_dim=32, intermediate_size=200,
               max_position_embeddings=256, bos_token_id=1, eos_token_id=380, rms_norm_eps=1e-5,
               rope_theta=1000000.0, tie_word_embeddings=False)
+# head size 128 (the matrix-core attention kernels in bfloat16), for contexts of thousands of
+# tokens; `max_position_embeddings` may be raised by the caller
+LONG = dict(vocab_size=1003, hidden_size=256, num_hidden_layers=2, num_attention_heads=8,
+            num_key_value_heads=4, head_dim=128, intermediate_size=640,
+            max_position_embeddings=5120, bos_token_id=0, eos_token_id=1, rms_norm_eps=1e-6,
+            rope_theta=1000000.0, tie_word_embeddings=False)
 SEEDS = {"A": 0, "B": 1}
 CONFIGS = {"A": TINY_A, "B": TINY_B}
 
@@ -41,6 +47,23 @@ def make_folder(name, root):
     path = Path(root) / f"tiny_{name}"
     if not (path / "model.safetensors").is_file():
         write_model_folder(path, tiny_config(name), SEEDS[name])
+    return path
+
+
+def make_long_folder(root, seed=3, head_norm_scale=1.5, **overrides):
+    """A model folder of the `LONG` shape whose q/k norm weights are raised by
+    `head_norm_scale`: that more than doubles the scores, so attention is peaked, and a key
+    that is left out, read twice or read from a foreign page moves the logits by far more
+    than the tolerance."""
+    from safetensors.torch import load_file, save_file
+    from edge_infer_amd import Qwen3Config, write_model_folder
+    path = Path(root) / "long_model"
+    write_model_folder(path, Qwen3Config(**dict(LONG, **overrides)), seed=seed)
+    tensors = load_file(str(path / "model.safetensors"))
+    for name in tensors:
+        if name.endswith("q_norm.weight") or name.endswith("k_norm.weight"):
+            tensors[name] = (tensors[name].float() * head_norm_scale).to(torch.bfloat16)
+    save_file(tensors, str(path / "model.safetensors"))
     return path
 
 

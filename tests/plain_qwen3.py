@@ -89,13 +89,15 @@ def rope(x, positions, theta):
     return torch.cat([first * cos - second * sin, first * sin + second * cos], dim=-1)
 
 
-def attention(q, k, v, positions=None, window=None):
+def attention(q, k, v, positions=None, window=None, key_positions=None):
     """Causal grouped-query attention of one sequence.
 
     q [S, nq, d], k and v [S, nkv, d]; query head h reads kv head
     h // (nq // nkv); scores scaled by 1/sqrt(d); key t is visible to the query
     at absolute position p iff t <= p (and t > p - window when a window is
     given; the reference has no window).  Softmax over visible keys.
+    `key_positions`: where the keys sit when q holds only some rows of the sequence
+    (then `positions` are those rows' places); by default the queries' own places.
 
     operators/src/cuda/execution.cu:137-179 (attention_scalar_kernel),
     runtime/src/qwen.cpp:374-402.
@@ -109,7 +111,8 @@ def attention(q, k, v, positions=None, window=None):
     positions = torch.as_tensor(positions, dtype=torch.long)
     out = torch.zeros(S, nq, d, dtype=F64)
     scale = 1.0 / math.sqrt(d)
-    key_pos = positions  # keys of a whole sequence sit at the same positions
+    # keys of a whole sequence sit at the same positions as its queries
+    key_pos = positions if key_positions is None else torch.as_tensor(key_positions, dtype=torch.long)
     for h in range(nq):
         g = h // group
         scores = (q[:, h, :] @ k[:, g, :].T) * scale  # [S, S]
@@ -142,12 +145,14 @@ def swiglu(gate, up):
 # ----------------------------------------------------------------------------
 # block and model
 # ----------------------------------------------------------------------------
-def attention_block(x, w, cfg, layer, positions):
+def attention_block(x, w, cfg, layer, positions, rows=None):
     """RMSNorm -> q/k/v -> per-head q/k RMSNorm -> RoPE -> attention -> o.
 
     runtime/include/execution/decoder.hpp:121-158; the per-head norm comes
     before the rotation (:125-136) and uses the model's one eps.  Each projection takes
     a bias when the checkpoint holds one (runtime/include/models/qwen3_model.hpp:386-395).
+    `rows`: the output for these rows of x only (keys and values of every row are still
+    made); what makes sequences of tens of thousands of tokens affordable.
     """
     p = f"model.layers.{layer}."
     S = x.shape[0]
@@ -162,8 +167,13 @@ def attention_block(x, w, cfg, layer, positions):
     k = rms_norm(k, w[p + "self_attn.k_norm.weight"], cfg["rms_norm_eps"])
     q = rope(q, positions, cfg["rope_theta"])
     k = rope(k, positions, cfg["rope_theta"])
-    a = attention(q, k, v, positions)
-    return linear(a.reshape(S, nq * d), w[p + "self_attn.o_proj.weight"],
+    if rows is None:
+        a = attention(q, k, v, positions)
+    else:
+        rows = torch.as_tensor(rows, dtype=torch.long)
+        a = attention(q[rows], k, v, torch.as_tensor(positions, dtype=torch.long)[rows],
+                      key_positions=positions)
+    return linear(a.reshape(a.shape[0], nq * d), w[p + "self_attn.o_proj.weight"],
                   w.get(p + "self_attn.o_proj.bias"))
 
 
@@ -195,17 +205,25 @@ def head_weight(w, cfg):
     raise KeyError("lm_head.weight")
 
 
-def forward(w, cfg, ids, positions=None):
+def forward(w, cfg, ids, positions=None, rows=None):
     """Logits [S, V] (float64) of one whole sequence.
 
     runtime/include/execution/decoder.hpp:119-169, runtime/src/qwen3.cpp:293-299.
+    `rows` (models of one layer only, whose rows need nothing of each other beyond the
+    layer's keys and values): logits [len(rows), V] at these places.
     """
     S = len(ids)
     if positions is None:
         positions = list(range(S))
     x = embedding(ids, w["model.embed_tokens.weight"])
+    if rows is not None and cfg["num_hidden_layers"] != 1:
+        raise ValueError("single rows can be asked of a model of one layer only")
     for layer in range(cfg["num_hidden_layers"]):
-        x = x + attention_block(x, w, cfg, layer, positions)
+        if rows is None:
+            x = x + attention_block(x, w, cfg, layer, positions)
+        else:
+            x = x[torch.as_tensor(rows, dtype=torch.long)] \
+                + attention_block(x, w, cfg, layer, positions, rows=rows)
         x = x + feed_forward_block(x, w, cfg, layer)
     y = rms_norm(x, w["model.norm.weight"], cfg["rms_norm_eps"])
     return linear(y, head_weight(w, cfg), w.get("lm_head.bias"))   # qwen3_model.hpp:371-372

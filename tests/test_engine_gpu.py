@@ -658,17 +658,20 @@ def test_a_failed_step_leaves_the_session_as_it_was_and_a_failed_wait_ends_it(mo
     torch.cuda.synchronize()
 
 
-# What the bfloat16 engine may differ by from the float32 engine on eight layers of the 8B
-# shape with the real vocabulary.  Measured on an MI355X: rms 0.0174, max 0.0211, 73.5 % of
-# the logits within the reference's bound, the same top token at 90.6 % of the places (about
-# 0.2 % of rounding error per operation, ten roundings a layer, adding up like a random walk).
-DEPTH_RMS_REL = 0.02          # root-mean-square difference / root-mean-square logit
-DEPTH_MAX_REL = 0.03          # largest difference / largest logit
-DEPTH_WITHIN_REFERENCE_BOUND = 0.70   # share of logits within the reference's bound, below
-DEPTH_SAME_TOP_TOKEN = 0.85   # share of places with the same most likely token
+# What the bfloat16 engine may differ by from the float32 engine on 8 and on all 36 layers of
+# the 8B shape with the real vocabulary: root-mean-square difference / root-mean-square logit,
+# largest difference / largest logit, the share of logits within the reference's bound (below)
+# and the share of places with the same most likely token.  Measured on an MI355X at 8 layers:
+# 0.0173, 0.0197, 73.7 %, 92.2 % (about 0.2 % of rounding error per operation, ten roundings a
+# layer, adding up like a random walk: the square root of the depth); at 36 layers: 0.0358,
+# 0.0417, 42.9 %, 96.9 %.  Random weights give logits of at most 0.6, so the absolute part of
+# the reference's bound, made for trained weights, decides less the deeper the model is.
+DEPTH_BOUNDS = {8: (0.02, 0.03, 0.70, 0.85),
+                36: (0.042, 0.05, 0.38, 0.85)}
 
 
-def test_bfloat16_against_float32_on_eight_layers_of_the_8b_shape():
+@pytest.mark.parametrize("layers", [8, 36])
+def test_bfloat16_against_float32_at_depth_on_the_8b_shape(layers):
     """The two precisions of the whole engine at real width and vocabulary, deeper than
     the tiny models: 300- and 120-token prompts, then 24 tokens one by one each.  Reported
     and bounded: rms and largest difference, the share of logits within the reference's
@@ -678,7 +681,7 @@ def test_bfloat16_against_float32_on_eight_layers_of_the_8b_shape():
     so equal top tokens everywhere cannot be asked for; where they differ the float32
     engine's own margin between the two must be small."""
     import edge_infer_amd as ei
-    cfg = ei.Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=8,
+    cfg = ei.Qwen3Config(vocab_size=151936, hidden_size=4096, num_hidden_layers=layers,
                          num_attention_heads=32, num_key_value_heads=8, head_dim=128,
                          intermediate_size=12288, max_position_embeddings=1024, bos_token_id=0,
                          eos_token_id=151645, rms_norm_eps=1e-6, rope_theta=1e6,
@@ -707,10 +710,11 @@ def test_bfloat16_against_float32_on_eight_layers_of_the_8b_shape():
     worst = diff.max().item() / exact.abs().max().item()
     within = (diff <= 0.015625 + 0.01 * torch.maximum(low.abs(), exact.abs())).double().mean().item()
     same = (low.argmax(-1) == exact.argmax(-1)).double().mean().item()
-    print(f"\nbfloat16 against float32, 8 layers of the 8B shape: rms {rms:.4f}, max {worst:.4f}, "
-          f"within the reference's bound {within:.4f}, same top token {same:.3f}")
-    assert rms <= DEPTH_RMS_REL and worst <= DEPTH_MAX_REL
-    assert within >= DEPTH_WITHIN_REFERENCE_BOUND and same >= DEPTH_SAME_TOP_TOKEN
+    print(f"\nbfloat16 against float32, {layers} layers of the 8B shape: rms {rms:.4f}, "
+          f"max {worst:.4f}, within the reference's bound {within:.4f}, same top token {same:.3f}")
+    rms_bound, max_bound, within_bound, same_bound = DEPTH_BOUNDS[layers]
+    assert rms <= rms_bound and worst <= max_bound
+    assert within >= within_bound and same >= same_bound
     # where the top token differs, float32 itself holds the two within bfloat16's error
     for row in (low.argmax(-1) != exact.argmax(-1)).nonzero().flatten().tolist():
         margin = exact[row].max() - exact[row, low[row].argmax()]
@@ -820,25 +824,26 @@ def test_steady_decoding_allocates_nothing_on_the_device(folders, tmp_path, dtyp
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_prompts_in_portions_give_the_logits_of_whole_prompts(tmp_path, dtype):
     """The generation loop's prompt steps under a row budget of 64: a prompt cut at 64 and
-    128, a portion of 2 tokens, requests that are left out of a step, at head size 64 (the
-    matrix-core kernels in bfloat16), against whole prompts in the plain implementation."""
+    128, a portion of 2 tokens that begins a page (positions 64 and 65), requests that are
+    left out of a step, at head size 64 (the matrix-core kernels in bfloat16), against whole
+    prompts in the plain implementation."""
     import edge_infer_amd as ei
     from edge_infer_amd.engine.generate import Request, _prefill, prompt_steps
     folder = head64_folder(tmp_path)
     cfg, w = plain.read_folder(folder)
-    prompts = [random_ids(500, n, 30 + n) for n in (70, 5, 130, 33, 52)]
+    prompts = [random_ids(500, n, 30 + n) for n in (66, 5, 130, 33, 52)]
     session = ei.Session(ei.load_model(folder, dtype=dtype), max_tokens=8 * 192, max_seqs=5)
     requests = [Request(prompt=p, limit=200, stream=i) for i, p in enumerate(prompts)]
     portions = [[(r.stream, first, count) for r, first, count, _ in step]
                 for step in prompt_steps(requests, 64)]
-    assert portions == [[(0, 0, 64)], [(0, 64, 6), (1, 0, 5), (2, 0, 53)], [(2, 53, 64)],
-                        [(2, 117, 13), (3, 0, 33), (4, 0, 18)], [(4, 18, 34)]]
+    assert portions == [[(0, 0, 64)], [(0, 64, 2), (1, 0, 5), (2, 0, 57)], [(2, 57, 64)],
+                        [(2, 121, 9), (3, 0, 33), (4, 0, 22)], [(4, 22, 30)]]
     for request in requests:
         request.slot = session.begin()
     logits = _prefill(session, requests, 64)
     expected = torch.stack([plain.forward(w, cfg, p)[-1] for p in prompts])
     assert_close(dtype, logits, expected, f"{dtype} prompts in portions")
-    assert [session.length(r.slot) for r in requests] == [70, 5, 130, 33, 52]
+    assert [session.length(r.slot) for r in requests] == [66, 5, 130, 33, 52]
     # and through the whole loop: the same tokens as with one prompt step
     session.reset()
     few = session.generate_batch(prompts, max_new_tokens=5, temperature=0.0, stop_ids=(),

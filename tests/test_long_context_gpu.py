@@ -11,29 +11,16 @@ import pytest
 import torch
 
 import plain_qwen3 as plain
-from helpers import assert_close_long as assert_close, random_ids
+from helpers import LONG, assert_close_long as assert_close, make_long_folder, random_ids
 
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LONG = dict(vocab_size=1003, hidden_size=256, num_hidden_layers=2, num_attention_heads=8,
-            num_key_value_heads=4, head_dim=128, intermediate_size=640,
-            max_position_embeddings=5120, bos_token_id=0, eos_token_id=1, rms_norm_eps=1e-6,
-            rope_theta=1000000.0, tie_word_embeddings=False)
 
 
 @pytest.fixture(scope="module")
 def folder(tmp_path_factory):
-    from safetensors.torch import load_file, save_file
-    import edge_infer_amd as ei
-    path = tmp_path_factory.mktemp("long") / "model"
-    ei.write_model_folder(path, ei.Qwen3Config(**LONG), seed=3)
-    tensors = load_file(str(path / "model.safetensors"))
-    for name in tensors:
-        if name.endswith("q_norm.weight") or name.endswith("k_norm.weight"):
-            tensors[name] = (tensors[name].float() * 1.5).to(torch.bfloat16)
-    save_file(tensors, str(path / "model.safetensors"))
-    return path
+    return make_long_folder(tmp_path_factory.mktemp("long"))
 
 
 @pytest.fixture(scope="module")
@@ -72,15 +59,16 @@ def test_a_prompt_of_4500_tokens_whole(models, oracle, dtype):
     session = ei.Session(models(dtype), max_tokens=4608, max_seqs=1)
     for tensor in session.cache.kv_k + session.cache.kv_v:
         tensor.fill_(float("nan"))
-    places = sorted({0, 1, 63, 64, 65, 1023, 1024, 2047, 2048, 4095, 4096, 4499,
+    places = sorted({0, 1, 63, 64, 65, 1023, 1024, 1499, 1500, 1501, 1502, 2047, 2048, 4095, 4096, 4499,
                      *range(7, 4500, 211)})
     slot = session.begin()
     logits = session.step([(slot, ids, places)])
     assert_close(dtype, logits, oracle(ids)[places], f"{dtype} 4,500 tokens whole")
-    # the same sequence in three portions of unequal size gives the same rows
+    # the same sequence in three portions of unequal size, the middle one of two tokens (the
+    # smallest item of the prompt path), gives the same rows
     session.end(slot)
     slot = session.begin()
-    cuts = [0, 1500, 1501, 4500]
+    cuts = [0, 1500, 1502, 4500]
     rows = []
     for begin, end in zip(cuts, cuts[1:]):
         want = [p - begin for p in places if begin <= p < end]

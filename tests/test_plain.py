@@ -294,3 +294,169 @@ def test_linear_bias_is_added_to_every_row():
     expected = torch.nn.functional.linear(x, w, b)
     assert torch.allclose(plain.linear(x, w, b), expected, atol=1e-12)
     assert torch.allclose(plain.linear(x, w, b) - plain.linear(x, w), b.expand(5, 3), atol=1e-12)
+
+
+# ----------------------------------------------------------------------------
+# the composition: what fixes the order of the parts beside the reference's text
+# ----------------------------------------------------------------------------
+def _wide_head_norms(w, cfg, seed):
+    """q/k norm weights far from 1 and different in the two halves of every rotation pair:
+    only then does their place relative to the rotation show."""
+    g = torch.Generator().manual_seed(seed)
+    d = plain.head_dim_of(cfg)
+    for i in range(cfg["num_hidden_layers"]):
+        for name in ("q_norm", "k_norm"):
+            w[f"model.layers.{i}.self_attn.{name}.weight"] = \
+                (0.4 + 2.0 * torch.rand(d, generator=g)).double()
+    return w
+
+
+def _attention_block_with_the_norm_after_the_rotation(x, w, cfg, layer, positions):
+    """The mistake that the shift test below must catch: rotation first, head norm second."""
+    p = f"model.layers.{layer}."
+    S = x.shape[0]
+    nq, nkv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], plain.head_dim_of(cfg)
+    h = plain.rms_norm(x, w[p + "input_layernorm.weight"], cfg["rms_norm_eps"])
+    q = plain.linear(h, w[p + "self_attn.q_proj.weight"]).reshape(S, nq, d)
+    k = plain.linear(h, w[p + "self_attn.k_proj.weight"]).reshape(S, nkv, d)
+    v = plain.linear(h, w[p + "self_attn.v_proj.weight"]).reshape(S, nkv, d)
+    q = plain.rms_norm(plain.rope(q, positions, cfg["rope_theta"]),
+                       w[p + "self_attn.q_norm.weight"], cfg["rms_norm_eps"])
+    k = plain.rms_norm(plain.rope(k, positions, cfg["rope_theta"]),
+                       w[p + "self_attn.k_norm.weight"], cfg["rms_norm_eps"])
+    a = plain.attention(q, k, v, positions)
+    return plain.linear(a.reshape(S, nq * d), w[p + "self_attn.o_proj.weight"])
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_only_distances_count_because_the_head_norm_precedes_the_rotation(name, monkeypatch):
+    """A rotation commutes with nothing that weighs the two halves of a pair differently, so
+    with head norm weights far from 1 the logits are free of a common shift of all positions
+    only if the norm comes before the rotation (runtime/include/execution/decoder.hpp:125-136).
+    The same model with the two exchanged moves by a hundred times the bound."""
+    cfg = dict(CONFIGS[name])
+    w = _wide_head_norms(_random_weights(cfg, 21), cfg, 22)
+    # larger projections, so that attention is far from uniform and the keys matter
+    for key in list(w):
+        if "q_proj" in key or "k_proj" in key:
+            w[key] = w[key] * 8
+    ids = [5, 3, 8, 13, 2, 1, 34, 21, 7, 7, 19]
+    shift = [p + 57 for p in range(len(ids))]
+    logits = plain.forward(w, cfg, ids)
+    scale = logits.abs().max()
+    assert (plain.forward(w, cfg, ids, positions=shift) - logits).abs().max() < 1e-4 * scale
+    monkeypatch.setattr(plain, "attention_block", _attention_block_with_the_norm_after_the_rotation)
+    wrong = plain.forward(w, cfg, ids)
+    assert (plain.forward(w, cfg, ids, positions=shift) - wrong).abs().max() > 1e-2 * wrong.abs().max()
+
+
+def test_with_silent_blocks_the_model_is_embedding_final_norm_and_head():
+    """o_proj = down_proj = 0 in every layer: what is left is head(norm(E[ids]) * w), from
+    library routines.  Fails for a scaled embedding, a final norm without its weight or
+    applied to the head's output, a residual that is not carried through, or a bias that
+    does not exist."""
+    cfg = dict(CONFIGS["B"])
+    w = _random_weights(cfg, 5)
+    for key in list(w):
+        if "o_proj" in key or "down_proj" in key:
+            w[key] = torch.zeros_like(w[key])
+    ids = [7, 300, 12, 12, 0]
+    x = F.embedding(torch.tensor(ids), w["model.embed_tokens.weight"])
+    y = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + cfg["rms_norm_eps"]) * w["model.norm.weight"]
+    assert torch.allclose(plain.forward(w, cfg, ids), F.linear(y, w["lm_head.weight"]), atol=1e-12)
+
+
+def _dominant_attention_model(seed):
+    """One layer, one head, made so that the feed-forward's input shows where its norm sits.
+
+    Every row of v_proj is the same vector, so attention's output is a scalar times (1,..,1);
+    o_proj sends that to s * scalar * e_0 with s = 1e9, which buries the embedding: the
+    residual after attention points along +-e_0 at every position, whatever the token.  The
+    second norm of a sequential block therefore hands the feed-forward +-sqrt(H) w2[0] e_0,
+    the same input (up to the sign) at every position.  down_proj writes with the same scale
+    s and never into coordinate 0; the head is the identity and the final norm's weight 1, so
+    the logits are the normalised residual and their part beyond coordinate 0 points along
+    the feed-forward's output."""
+    cfg = dict(vocab_size=24, hidden_size=24, num_hidden_layers=1, num_attention_heads=1,
+               num_key_value_heads=1, head_dim=16, intermediate_size=40, rms_norm_eps=1e-30,
+               rope_theta=1e4, tie_word_embeddings=False, eos_token_id=23)
+    w = _random_weights(cfg, seed)
+    H, d, s = cfg["hidden_size"], 16, 1e9
+    p = "model.layers.0."
+    w[p + "self_attn.v_proj.weight"] = w[p + "self_attn.v_proj.weight"][:1].expand(d, H).clone()
+    o = torch.zeros(H, d, dtype=torch.float64)
+    o[0, :] = s / d
+    w[p + "self_attn.o_proj.weight"] = o
+    down = w[p + "mlp.down_proj.weight"] * s * 10
+    down[0, :] = 0
+    w[p + "mlp.down_proj.weight"] = down
+    w[p + "mlp.gate_proj.weight"] = w[p + "mlp.gate_proj.weight"] * 10
+    w["model.norm.weight"] = torch.ones(H, dtype=torch.float64)
+    w["lm_head.weight"] = torch.eye(H, dtype=torch.float64)
+    return cfg, w
+
+
+def test_the_second_norm_reads_the_residual_after_attention_was_added():
+    """runtime/include/execution/decoder.hpp:159-161: the feed-forward's norm reads the sum.
+    In the model above its output is then one of two vectors, from library routines:
+    down(silu(c gate[:, 0]) * c up[:, 0]) with c = +-sqrt(H) w2[0].  A block whose second
+    norm read the residual before attention's addition (or the embedding) would give a
+    different direction at every position."""
+    cfg, w = _dominant_attention_model(13)
+    p = "model.layers.0."
+    ids = [3, 17, 9, 21, 0, 11, 5, 5, 14]
+    logits = plain.forward(w, cfg, ids)
+    H = cfg["hidden_size"]
+    c = math.sqrt(H) * w[p + "post_attention_layernorm.weight"][0]
+    candidates = []
+    for sign in (1.0, -1.0):
+        hidden = F.silu(sign * c * w[p + "mlp.gate_proj.weight"][:, 0]) \
+            * (sign * c * w[p + "mlp.up_proj.weight"][:, 0])
+        delta = F.linear(hidden, w[p + "mlp.down_proj.weight"])[1:]
+        candidates.append(delta / delta.norm())
+    assert (candidates[0] - candidates[1]).norm() > 0.1     # the two signs are told apart
+    seen = set()
+    for row in logits:
+        direction = row[1:] / row[1:].norm()
+        errors = [(direction - candidate).norm().item() for candidate in candidates]
+        assert min(errors) < 1e-6, errors
+        seen.add(errors.index(min(errors)))
+    # the rows' own embeddings differ, so a norm that read them would not give one direction
+    x0 = w["model.embed_tokens.weight"][torch.tensor(ids)]
+    assert (x0[0] / x0[0].norm() - x0[1] / x0[1].norm()).norm() > 0.1
+
+
+def test_the_second_norm_test_tells_a_parallel_block_apart(monkeypatch):
+    """The check above is not empty: with a block whose feed-forward reads the residual as it
+    was before attention (x + attn(n1 x) + ffn(n2 x)) the rows' directions scatter."""
+    cfg, w = _dominant_attention_model(13)
+    ids = [3, 17, 9, 21, 0, 11, 5, 5, 14]
+    before = {}
+    real_attention, real_feed_forward = plain.attention_block, plain.feed_forward_block
+
+    def attention_block(x, *args):
+        before["x"] = x
+        return real_attention(x, *args)
+
+    def feed_forward_block(x, *args):
+        return real_feed_forward(before["x"], *args)
+
+    monkeypatch.setattr(plain, "attention_block", attention_block)
+    monkeypatch.setattr(plain, "feed_forward_block", feed_forward_block)
+    logits = plain.forward(w, cfg, ids)
+    directions = torch.stack([row[1:] / row[1:].norm() for row in logits])
+    spread = (directions[:, None, :] - directions[None, :, :]).norm(dim=-1)
+    pairs_apart = ((spread > 0.1) & ((directions[:, None, :] + directions[None, :, :]).norm(dim=-1) > 0.1))
+    assert pairs_apart.sum() > len(ids)
+
+
+def test_single_rows_of_a_one_layer_model_are_the_rows_of_the_whole():
+    """The rows-only form that the tests of long contexts use."""
+    cfg = dict(CONFIGS["B"], num_hidden_layers=1)
+    w = _random_weights(cfg, 31)
+    ids = [(7 * i + 3) % cfg["vocab_size"] for i in range(41)]
+    whole = plain.forward(w, cfg, ids)
+    rows = [0, 1, 17, 39, 40, 17]
+    assert torch.allclose(plain.forward(w, cfg, ids, rows=rows), whole[rows], atol=1e-12)
+    with pytest.raises(ValueError):
+        plain.forward(_random_weights(dict(CONFIGS["B"]), 31), dict(CONFIGS["B"]), ids, rows=[0])
