@@ -13,8 +13,12 @@ headline batch without HIP graphs.
 `--only generate` times the generation loop instead: a batch of prompts with lengths
 uniform in [64, 2048] that start together, then `--new-tokens` greedy tokens each (the
 workload named for the 0.6B shape, with `--shape 0.6b --batch 32 --context 8192`).
-`points` also hold the generation workload of the 0.6B shape (its decode step and its
-prompt step) and, with `--with-32b`, decode at batch 1 and 16 and the prefill of the 32B shape.
+`points` also hold the generation workload of the 0.6B shape (the whole loop, its decode
+steps timed as steps, its prompt step) and decode at batch 1 and 16 and the prefill of the
+32B shape (`--without-32b` leaves those out).  `points` is flat: beside every rate `<name>`
+stand `<name>_ms` (a step), `<name>_GB` (what the step has to read, or `_TFLOP`: what it has
+to multiply), `<name>_frac` (of the published peak) and `<name>_frac_measured` (of what the
+chip at hand gives).
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
 a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
@@ -54,22 +58,39 @@ def model_config(shape, layers):
                           rope_theta=1e6, tie_word_embeddings=tied)
 
 
-def step_bytes(cfg, batch, context, itemsize):
-    """Bytes a decode step has to read: layer and head weights once, the live cache."""
+def step_bytes(cfg, cached_tokens, itemsize):
+    """Bytes a decode step has to read: layer and head weights once, and the keys and values
+    of the `cached_tokens` tokens that its live requests hold together."""
     H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
     layer = (Q + 2 * KV) * H + H * Q + 3 * I * H
     weights = itemsize * (cfg.num_hidden_layers * layer + V * H)
-    cache = itemsize * 2 * cfg.num_hidden_layers * KV * batch * context
+    cache = itemsize * 2 * cfg.num_hidden_layers * KV * cached_tokens
     return weights + cache
 
 
-def prefill_flops(cfg, tokens):
+def prefill_flops(cfg, lengths):
+    """Floating-point operations of one prompt step over prompts of these lengths, each
+    wanting the logits of its last token."""
+    if isinstance(lengths, int):
+        lengths = [lengths]
     H, I, V = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
     Q, KV = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    tokens = sum(lengths)
     layer = 2 * tokens * ((Q + 2 * KV) * H + H * Q + 3 * I * H)
-    attention = 2 * 2 * cfg.num_attention_heads * cfg.head_dim * tokens * (tokens + 1) / 2
-    return cfg.num_hidden_layers * (layer + attention) + 2 * V * H
+    attention = sum(2 * 2 * cfg.num_attention_heads * cfg.head_dim * n * (n + 1) / 2
+                    for n in lengths)
+    return cfg.num_hidden_layers * (layer + attention) + len(lengths) * 2 * V * H
+
+
+def unequal_prompts(cfg, batch, seed=5):
+    """Prompts with lengths uniform in [64, 2048], the generation workload's."""
+    import random
+    import torch
+    rng = random.Random(seed)
+    lengths = [rng.randint(64, 2048) for _ in range(batch)]
+    g = torch.Generator().manual_seed(1)
+    return [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lengths]
 
 
 def synthetic_prompts(cfg, batch, length, seed):
@@ -78,8 +99,11 @@ def synthetic_prompts(cfg, batch, length, seed):
     return torch.randint(0, cfg.vocab_size, (batch, length), generator=g).tolist()
 
 
-def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True, context=CONTEXT):
-    """(mean ms per step, mean context during the timed steps, median ms per step)."""
+def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True, context=CONTEXT,
+                   prompts=None):
+    """(mean ms per step, mean context of a sequence during the timed steps, median ms per
+    step).  `prompts`: the batch's prompts (of unequal lengths, say) instead of `batch`
+    synthetic ones of `prompt` tokens; the mean context is then the mean over them."""
     import torch
     import edge_infer_amd as ei
     from edge_infer_amd.sampling import Sampler, SamplingParams
@@ -87,9 +111,11 @@ def measure_decode(model, cfg, batch, steps, warmup, prompt=PROMPT, graphs=True,
                          max_seq_tokens=context, graphs=graphs)
     sampler = Sampler(model.device)
     greedy = SamplingParams(temperature=0.0)
-    prompts = synthetic_prompts(cfg, batch, prompt, seed=100 + batch)
+    if prompts is None:
+        prompts = synthetic_prompts(cfg, batch, prompt, seed=100 + batch)
+    prompt = sum(len(p) for p in prompts) / len(prompts)
     slots = [session.begin() for _ in range(batch)]
-    logits = session.step([(s, p, [prompt - 1]) for s, p in zip(slots, prompts)], copy=False)
+    logits = session.step([(s, p, [len(p) - 1]) for s, p in zip(slots, prompts)], copy=False)
     tokens = sampler(logits, greedy, [], [])
     stamps = []
 
@@ -140,13 +166,10 @@ def measure_prefill(model, cfg, repeats=3, tokens=PREFILL_TOKENS):
 def measure_generate(model, cfg, batch, context, new_tokens, repeats=2):
     """Best wall time of `Session.generate_batch` over a batch of unequal prompts, and the
     time of its prompt step alone."""
-    import random
     import torch
     import edge_infer_amd as ei
-    rng = random.Random(5)
-    lengths = [rng.randint(64, 2048) for _ in range(batch)]
-    g = torch.Generator().manual_seed(1)
-    prompts = [torch.randint(0, cfg.vocab_size, (n,), generator=g).tolist() for n in lengths]
+    prompts = unequal_prompts(cfg, batch)
+    lengths = [len(p) for p in prompts]
     session = ei.Session(model, max_tokens=batch * context, max_seqs=batch,
                          max_seq_tokens=context)
     total = None
@@ -166,7 +189,9 @@ def measure_generate(model, cfg, batch, context, new_tokens, repeats=2):
     prompt_s = time.perf_counter() - started
     for s in slots:
         session.end(s)
-    return total, prompt_s, sum(lengths), sum(len(o) for o in out)
+    del session
+    torch.cuda.empty_cache()
+    return total, prompt_s, lengths, sum(len(o) for o in out)
 
 
 def measure_peaks():
@@ -204,30 +229,63 @@ def data_bytes_of(gib):
     return gib * 1024 ** 3
 
 
-def other_shape_points(args):
+def decode_point(points, name, cfg, batch, ms, cached_tokens, itemsize, peaks):
+    """A decode measurement as flat entries of `points`: tokens a second, a step's time, what
+    it has to read, and the fractions of the published and of the measured read rate."""
+    nbytes = step_bytes(cfg, cached_tokens, itemsize)
+    rate = nbytes / (ms * 1e-3) / 1e9
+    points[name] = round(batch * 1000.0 / ms, 1)
+    points[name + "_ms"] = round(ms, 4)
+    points[name + "_GB"] = round(nbytes / 1e9, 3)
+    points[name + "_frac"] = round(rate / HBM_PEAK_GBS, 4)
+    points[name + "_frac_measured"] = round(rate / peaks["hbm_read_GBs"], 4)
+
+
+def prefill_point(points, name, cfg, lengths, ms, dtype, peaks):
+    """A prompt step the same way: tokens a second, its time, its operations, fractions of the
+    published and of the measured matrix-core rate."""
+    flops = prefill_flops(cfg, lengths)
+    tokens = lengths if isinstance(lengths, int) else sum(lengths)
+    points[name] = round(tokens * 1000.0 / ms, 1)
+    points[name + "_ms"] = round(ms, 3)
+    points[name + "_TFLOP"] = round(flops / 1e12, 3)
+    points[name + "_frac"] = round(flops / (ms * 1e-3) / (PEAK_TFLOPS[dtype] * 1e12), 4)
+    if dtype == "bfloat16":
+        points[name + "_frac_measured"] = round(flops / (ms * 1e-3)
+                                                / (peaks["mfma_bf16_TFLOPs"] * 1e12), 4)
+
+
+def other_shape_points(args, itemsize, peaks):
     """Decode and prefill figures of the other shapes, as flat numbers for `points`."""
     import torch
     import edge_infer_amd as ei
     points = {}
     cfg = model_config("0.6b", 0)
     model = ei.random_model(cfg, seed=3, dtype=args.dtype)
-    total, prompt_s, prompt_tokens, new = measure_generate(model, cfg, 32, 8192, 256, repeats=1)
+    batch, new_tokens = 32, 256
+    total, prompt_s, lengths, new = measure_generate(model, cfg, batch, 8192, new_tokens, repeats=1)
     points["gen_0.6b_b32_new_tokens_per_s"] = round(new / total, 1)
-    points["gen_0.6b_b32_ms_per_decode_step"] = round(1e3 * (total - prompt_s) / 255, 4)
-    points["gen_0.6b_b32_prompt_tokens_per_s"] = round(prompt_tokens / prompt_s, 1)
+    points["gen_0.6b_b32_total_ms"] = round(1e3 * total, 1)
+    prefill_point(points, "gen_0.6b_b32_prompt_tokens_per_s", cfg, lengths, 1e3 * prompt_s,
+                  args.dtype, peaks)
+    # the loop's decode steps, timed as steps: the same prompts, then 255 tokens each, all but
+    # the first four timed (the mean holds the steps that capture a graph for a new context
+    # bound, as the loop's own time does; the median does not)
+    ms, context, median = measure_decode(model, cfg, batch, new_tokens - 5, 4, context=8192,
+                                         prompts=unequal_prompts(cfg, batch))
+    decode_point(points, "gen_0.6b_b32_decode", cfg, batch, ms, batch * context, itemsize, peaks)
+    points["gen_0.6b_b32_decode_ms_median"] = round(median, 4)
     del model
     torch.cuda.empty_cache()
-    if args.with_32b:
+    if not args.without_32b:
         cfg = model_config("32b", 0)
         model = ei.random_model(cfg, seed=4, dtype=args.dtype)
         for batch in (1, 16):
-            ms, _, median = measure_decode(model, cfg, batch, 16, 4)
-            points[f"32b_decode_b{batch}"] = round(batch * 1000.0 / ms, 1)
-            points[f"32b_decode_b{batch}_ms_median"] = round(median, 4)
+            ms, context, _ = measure_decode(model, cfg, batch, 16, 4)
+            decode_point(points, f"32b_decode_b{batch}", cfg, batch, ms, batch * context,
+                         itemsize, peaks)
         ms = measure_prefill(model, cfg, repeats=2)
-        points["32b_prefill_tokens_per_s"] = round(PREFILL_TOKENS * 1000.0 / ms, 1)
-        points["32b_prefill_frac"] = round(prefill_flops(cfg, PREFILL_TOKENS) / (ms * 1e-3)
-                                           / (PEAK_TFLOPS[args.dtype] * 1e12), 4)
+        prefill_point(points, "32b_prefill_tokens_per_s", cfg, PREFILL_TOKENS, ms, args.dtype, peaks)
         del model
         torch.cuda.empty_cache()
     return points
@@ -256,8 +314,9 @@ def main():
     parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS,
                         help="with --only prefill: the length of the one prompt (the record's "
                              "prefill is always of 2,048 tokens)")
-    parser.add_argument("--with-32b", action="store_true",
-                        help="also measure the 32B shape (decode at batch 1 and 16, prefill)")
+    parser.add_argument("--with-32b", action="store_true", help="(the default; kept for old command lines)")
+    parser.add_argument("--without-32b", action="store_true",
+                        help="leave the 32B shape (decode at batch 1 and 16, prefill) out of `points`")
     parser.add_argument("--peaks", action="store_true",
                         help="measure the read and matrix-core yardsticks only")
     args = parser.parse_args()
@@ -280,15 +339,16 @@ def main():
     if args.only == "decode":
         ms_step, context, median = measure_decode(model, cfg, args.batch, args.steps, args.warmup,
                                                   args.prompt, context=max(CONTEXT, args.context))
-        rate = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9
+        rate = step_bytes(cfg, args.batch * context, itemsize) / (ms_step * 1e-3) / 1e9
         print(json.dumps({"only": "decode", "shape": args.shape, "batch": args.batch,
                           "ms_per_step": round(ms_step, 4), "ms_per_step_median": round(median, 4),
                           "tokens_per_s": round(args.batch * 1000.0 / ms_step, 1),
                           "context": round(context), "GB/s": round(rate, 1)}))
         return 0
     if args.only == "generate":
-        total, prompt_s, prompt_tokens, new = measure_generate(model, cfg, args.batch,
-                                                               args.context, args.new_tokens)
+        total, prompt_s, lengths, new = measure_generate(model, cfg, args.batch,
+                                                         args.context, args.new_tokens)
+        prompt_tokens = sum(lengths)
         steps = args.new_tokens - 1          # the first token comes from the prompt step
         print(json.dumps({"only": "generate", "shape": args.shape, "batch": args.batch,
                           "prompt_tokens": prompt_tokens, "new_tokens": new,
@@ -308,23 +368,24 @@ def main():
         return 0
     ms_step, context, median_step = measure_decode(model, cfg, args.batch, args.steps, args.warmup)
     value = args.batch * 1000.0 / ms_step
-    achieved = step_bytes(cfg, args.batch, context, itemsize) / (ms_step * 1e-3) / 1e9
+    achieved = step_bytes(cfg, args.batch * context, itemsize) / (ms_step * 1e-3) / 1e9
     prefill_ms = measure_prefill(model, cfg)
     flops = prefill_flops(cfg, PREFILL_TOKENS)
+    peaks = measure_peaks()
     points = {}
     if not args.skip_points:
         for name, batch in (("decode_b1", 1), ("decode_b64", 64)):
-            ms, _, _ = measure_decode(model, cfg, batch, max(8, args.steps // 2), args.warmup)
-            points[name] = round(batch * 1000.0 / ms, 1)
+            ms, at, _ = measure_decode(model, cfg, batch, max(8, args.steps // 2), args.warmup)
+            decode_point(points, name, cfg, batch, ms, batch * at, itemsize, peaks)
         # the headline batch with every kernel launched by the host instead of from a HIP graph
-        ms, _, _ = measure_decode(model, cfg, args.batch, max(8, args.steps // 2), args.warmup,
-                                  graphs=False)
-        points[f"decode_b{args.batch}_eager"] = round(args.batch * 1000.0 / ms, 1)
-    peaks = measure_peaks()
+        ms, at, _ = measure_decode(model, cfg, args.batch, max(8, args.steps // 2), args.warmup,
+                                   graphs=False)
+        decode_point(points, f"decode_b{args.batch}_eager", cfg, args.batch, ms, args.batch * at,
+                     itemsize, peaks)
     if not args.skip_points and args.shape == "8b":
         del model
         torch.cuda.empty_cache()
-        points.update(other_shape_points(args))
+        points.update(other_shape_points(args, itemsize, peaks))
     from edge_infer_amd.csrc import lib
     record = {
         "metric": f"decode tokens/s, Qwen3-{args.shape.upper()} shape, batch {args.batch} after "

@@ -78,6 +78,7 @@ _SIGNATURES = {
         "ei_argmax": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
         "ei_argmax_partial_size": [c_int, c_int],
         "ei_argmax_static": [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p],
+        "ei_argmax_static_prepare": [],
         "ei_sample": [c_void_p, c_int, c_int, c_float, c_float, c_int, c_ulonglong, c_void_p,
                       c_void_p, c_void_p, c_void_p, c_void_p, c_longlong, c_void_p],
         "ei_sample_scratch_size": [c_int, c_int],

@@ -537,8 +537,42 @@ static __device__ __align__(256) float2 argmax_static_scratch[EI_ARGMAX_STATIC_M
 constexpr int kStaticDevices = 64;
 static std::atomic<float2*> argmax_static_address[kStaticDevices];
 
-// See sampling_static.h.  The first call on a device looks the array's address up (with that
-// device current) and keeps it; nothing is allocated then or later.
+// The array's address on the current device: looked up once per device (with that device
+// current) and kept.  The lookup may load the library's code on the device, which a stream
+// that is being captured does not allow, so it is never started from a call under capture.
+static int argmax_static_resolve(float2** out, bool capturing) {
+  int device = -1;
+  hipError_t status = hipGetDevice(&device);
+  if (status != hipSuccess) {
+    ei_set_error(hipGetErrorString(status));
+    return static_cast<int>(status);
+  }
+  EI_REQUIRE(device >= 0 && device < kStaticDevices, "argmax_static: device index out of range");
+  float2* partial = argmax_static_address[device].load(std::memory_order_acquire);
+  if (partial == nullptr) {
+    EI_REQUIRE(!capturing, "argmax_static: the first call on a device cannot run under stream "
+                           "capture; call ei_argmax_static_prepare() on that device before");
+    void* address = nullptr;
+    status = hipGetSymbolAddress(&address, HIP_SYMBOL(argmax_static_scratch));
+    if (status != hipSuccess) {
+      ei_set_error(hipGetErrorString(status));
+      return static_cast<int>(status);
+    }
+    EI_REQUIRE(address != nullptr, "argmax_static: the static buffer has no device address");
+    partial = static_cast<float2*>(address);
+    argmax_static_address[device].store(partial, std::memory_order_release);
+  }
+  *out = partial;
+  return 0;
+}
+
+// See sampling_static.h.
+extern "C" int ei_argmax_static_prepare() {
+  float2* partial = nullptr;
+  return argmax_static_resolve(&partial, false);
+}
+
+// See sampling_static.h.  Nothing is allocated, by this call or by the lookup.
 extern "C" int ei_argmax_static(const float* logits, int rows, int V, int32_t* tokens,
                                 float* probabilities, hipStream_t stream) {
   EI_REQUIRE(rows > 0 && V > 0, "argmax_static: sizes must be positive");
@@ -551,25 +585,11 @@ extern "C" int ei_argmax_static(const float* logits, int rows, int V, int32_t* t
   EI_REQUIRE(static_cast<long long>(rows) * chunks <= EI_ARGMAX_STATIC_MAX_PARTIALS,
              "argmax_static: rows * ceil(V / 4096) exceeds the 65536 partial results that the "
              "library's static buffer holds");
-  int device = -1;
-  hipError_t status = hipGetDevice(&device);
-  if (status != hipSuccess) {
-    ei_set_error(hipGetErrorString(status));
-    return static_cast<int>(status);
-  }
-  EI_REQUIRE(device >= 0 && device < kStaticDevices, "argmax_static: device index out of range");
-  float2* partial = argmax_static_address[device].load(std::memory_order_acquire);
-  if (partial == nullptr) {
-    void* address = nullptr;
-    status = hipGetSymbolAddress(&address, HIP_SYMBOL(argmax_static_scratch));
-    if (status != hipSuccess) {
-      ei_set_error(hipGetErrorString(status));
-      return static_cast<int>(status);
-    }
-    EI_REQUIRE(address != nullptr, "argmax_static: the static buffer has no device address");
-    partial = static_cast<float2*>(address);
-    argmax_static_address[device].store(partial, std::memory_order_release);
-  }
+  hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
+  float2* partial = nullptr;
+  const int resolved = argmax_static_resolve(&partial, capture != hipStreamCaptureStatusNone);
+  if (resolved != 0) return resolved;
   argmax_chunks_kernel<<<dim3(static_cast<unsigned>(chunks), rows), kArgmaxThreads, 0, stream>>>(
       logits, V, partial);
   argmax_merge_kernel<<<rows, EI_WAVE, 0, stream>>>(partial, static_cast<int>(chunks), tokens,

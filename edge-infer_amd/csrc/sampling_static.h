@@ -26,9 +26,19 @@ extern "C" {
 // EI_ARGMAX_STATIC_MAX_PARTIALS.  The call allocates nothing and frees nothing; its kernels
 // run on `stream`.  Every call on a GPU shares that GPU's array (each call overwrites all
 // the entries it later reads, so nothing has to be cleared): calls that overlap in time on
-// one GPU, on different streams or from different threads, race.
+// one GPU, on different streams or from different threads, race; so do two replays of graphs
+// that hold this call.
+//
+// The first call on a device looks up the array's address there, which a stream under
+// capture does not allow: before capturing a call, run ei_argmax_static_prepare() (or one
+// call of ei_argmax_static itself) on that device outside any capture.  A first call under
+// capture is refused with an error and leaves the capture valid.
 int ei_argmax_static(const float* logits, int rows, int V, int32_t* tokens, float* probabilities,
                      hipStream_t stream);
+
+// Looks up the static array's address on the current device, once; allocates nothing.
+// Returns 0, or non-zero with a message in ei_last_error().
+int ei_argmax_static_prepare(void);
 
 #ifdef __cplusplus
 }

@@ -142,3 +142,36 @@ def test_a_batch_of_100_and_20000_tokens(models, oracle, dtype):
         assert_close(dtype, torch.stack(rows), oracle(request, range(n - 1, n + 8)),
                      f"{dtype} context {n} beside the other")
     assert session.graph_replays == 7
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_eight_like_prompts_take_paired_work_items(models, oracle, dtype, monkeypatch):
+    """Eight prompts of 2,048 tokens in one step: enough work items of like prompts for the
+    matrix-core prefill kernel to run one wave a key range (`key_ways` 1) and to give every
+    block a long item and a short one (`pair_items`), which a single prompt never reaches."""
+    import edge_infer_amd as ei
+    from edge_infer_amd.csrc import lib
+    seen = []
+    launch = lib.attention_prefill_mfma
+
+    def spy(*args, **kwargs):
+        seen.append((kwargs["key_ways"], kwargs["pair_items"], args[6]))
+        return launch(*args, **kwargs)
+    monkeypatch.setattr(lib, "attention_prefill_mfma", spy)
+    prompts = [ids_of(2048, seed=50 + i) for i in range(8)]
+    session = ei.Session(models(dtype), max_tokens=8 * 2048, max_seqs=8)
+    for tensor in session.cache.kv_k + session.cache.kv_v:
+        tensor.fill_(float("nan"))
+    slots = [session.begin() for _ in prompts]
+    places = [0, 1, 63, 64, 127, 128, 1000, 1023, 1024, 1919, 1920, 2046, 2047]
+    logits = session.step([(slot, prompt, places) for slot, prompt in zip(slots, prompts)])
+    for index, prompt in enumerate(prompts):
+        assert_close(dtype, logits[index * len(places):(index + 1) * len(places)],
+                     oracle(prompt, places), f"{dtype} prompt {index} of eight")
+    mixer = session.model.layers[0].mixer
+    if mixer.matrix_cores:
+        items = 8 * 2048 // mixer.positions_per_item(1)
+        assert mixer.prefill_key_ways([2048] * 8) == 1 and seen == [(1, True, items)]
+        assert items * mixer.spec.n_kv_heads >= 2 * mixer.compute_units     # the kernel pairs them
+    else:
+        assert not seen

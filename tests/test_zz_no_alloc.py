@@ -17,6 +17,8 @@ def sampling():
     handle.ei_argmax_static.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
                                         ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p]
     handle.ei_argmax_static.restype = ctypes.c_int
+    handle.ei_argmax_static_prepare.argtypes = []
+    handle.ei_argmax_static_prepare.restype = ctypes.c_int
     handle.ei_argmax.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
                                  ctypes.c_void_p, ctypes.c_void_p, ctypes.c_longlong,
                                  ctypes.c_void_p]
@@ -24,6 +26,9 @@ def sampling():
     handle.ei_argmax_partial_size.argtypes = [ctypes.c_int, ctypes.c_int]
     handle.ei_argmax_partial_size.restype = ctypes.c_int
     handle.ei_last_error.restype = ctypes.c_char_p
+    # the array's address is looked up once per device, outside any capture and before the
+    # driver's free memory is read below (the lookup may load the library's code)
+    assert handle.ei_argmax_static_prepare() == 0, handle.ei_last_error()
     return handle
 
 
@@ -51,12 +56,17 @@ def _both(sampling, logits):
     got = torch.full((rows,), -7, dtype=torch.int32, device="cuda")
     got_p = torch.zeros(rows, dtype=torch.float32, device="cuda")
     torch.cuda.synchronize()
-    before = torch.cuda.memory_stats()["allocation.all.allocated"]
+    # the driver's own count of free bytes: it sees an allocation by anyone in the process,
+    # which torch's statistics (its own allocator's only) would not
+    free_before, _ = torch.cuda.mem_get_info()
+    torch_before = torch.cuda.memory_stats()["allocation.all.allocated"]
     status = sampling.ei_argmax_static(logits.data_ptr(), rows, vocab, got.data_ptr(),
                                        got_p.data_ptr(), stream)
     assert status == 0, sampling.ei_last_error()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_stats()["allocation.all.allocated"] == before
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after >= free_before, f"{free_before - free_after} bytes were allocated"
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == torch_before
     return got.tolist(), want.tolist(), got_p.tolist(), want_p.tolist()
 
 
@@ -85,3 +95,29 @@ def test_sizes_beyond_the_static_buffer_are_refused(sampling):
     assert status != 0
     assert b"65536" in sampling.ei_last_error()
     assert sampling.ei_argmax_static(logits.data_ptr(), 0, vocab, tokens.data_ptr(), None, None) != 0
+
+
+def test_captured_in_a_graph_and_replayed(sampling):
+    """The call inside a stream capture (after the address was looked up outside one), then
+    replayed over changing logits, with eager work of the program between the replays; every
+    replay against the eager entry point."""
+    rows, vocab = 5, 151936
+    logits = _logits(rows, vocab, seed=4)
+    tokens = torch.full((rows,), -7, dtype=torch.int32, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        status = sampling.ei_argmax_static(logits.data_ptr(), rows, vocab, tokens.data_ptr(), None,
+                                           torch.cuda.current_stream().cuda_stream)
+    assert status == 0, sampling.ei_last_error()
+    for seed in (5, 6, 7, 8):
+        logits.copy_(_logits(rows, vocab, seed=seed))
+        tokens.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = tokens.tolist()
+        # eager work between the replays: the same search through the other entry point,
+        # and a smaller call of this one that leaves stale partial results behind
+        assert got == _both(sampling, logits)[0]
+        _both(sampling, _logits(2, 20000, seed=seed + 10))
+        assert got == logits.nan_to_num(nan=float("-inf")).argmax(dim=1).tolist()
