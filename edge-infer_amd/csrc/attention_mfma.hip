@@ -371,17 +371,28 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
 // (HB = 4, 2 or 1, the largest that divides the group) and 32 * (8 / HB) consecutive positions
 // of one sequence; a wave keeps 32 rows of one head as operands in registers and walks the key
 // pages of the sequence.  A page of keys and a page of values go to LDS once for the whole
-// block, so the heads of a group share every byte that is fetched; two pages alternate, so
-// that a page costs one barrier.  KW = 2: the eight waves are HB heads x half as many groups of
-// rows x 2 halves of every page's keys; the wave of the second half hands its maximum, sum and
-// output tile to the wave of the first through LDS at the end.  Work items are then half as
-// long, so a short prompt gives twice the blocks, enough for the pairing of a long item with a
-// short one below (one 2,048-token prompt of 32/8 heads: 72 against 82 us).  With enough blocks
-// without it KW = 1 is faster (what a page costs a wave beside its products is not halved).
-// (A form with 16-row waves on 16x16x32 products, four waves
-// a SIMD, was measured against this one: an operand read from LDS feeds half the arithmetic
-// there and the instruction itself runs at a lower rate on this chip, 1.45 against 2.1
-// PFLOP/s in a loop of nothing else; it was 20 % slower from 3,000 tokens on and equal below.)
+// block, so the heads of a group share every byte that is fetched.  KW = 2: the eight waves are
+// HB heads x half as many groups of rows x 2 halves of every page's keys; the wave of the
+// second half hands its maximum, sum and output tile to the wave of the first through LDS at
+// the end.  Work items are then half as long, so a short prompt gives twice the blocks, enough
+// for the pairing of a long item with a short one below.  With enough blocks without it KW = 1
+// is faster (what a page costs a wave beside its products is not halved).
+// (A form with 16-row waves on 16x16x32 products, four waves a SIMD, was measured against this
+// one: an operand read from LDS feeds half the arithmetic there and the instruction itself
+// runs at a lower rate on this chip, 1.45 against 2.1 PFLOP/s in a loop of nothing else; it
+// was 20 % slower from 3,000 tokens on and equal below.)
+//
+// Pages move from global memory straight into LDS (global_load_lds: a wave load lands as one
+// kilobyte, lane l's 16 bytes at place l of it; no staging registers, no LDS stores), three
+// page buffers in turn: while page p is multiplied, page p + 1 is on its way or there and page
+// p + 2 is requested into the buffer that page p - 1 left at the last barrier.  One barrier a
+// page says both that the next page is complete (every wave has waited for its own loads of
+// it) and that this one's buffer is free.  Both pages lie in LDS row by row as in the cache,
+// with the pieces of a row exchanged among themselves (below) so that operand reads meet
+// every bank once; a lane fetches the piece that belongs at its place.  The slots of a
+// sequence's last page beyond the item's last position hold whatever the cache held before:
+// their scores are masked, and their value rows are cleared in LDS by the wave that fetched
+// them (a probability of zero times a stale NaN would still be NaN).
 //
 // S^T = K Q^T for a block of 32 keys: A = keys (lane (key l % 32, half l / 32) reads
 // k[key][16 s + 8 half .. +8] from LDS), B = the wave's queries in registers (lane (query
@@ -389,26 +400,41 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
 // with keys 8 i + 4 h + r of the block (i, r = 0..3): for a 16-key step t of the value
 // product these are keys 16 t + 4 h + r and 16 t + 8 + 4 h + r, eight values that are
 // exactly the lane's A operand of P, provided the values (B, lane (d column n, half h)) come
-// in the same order: two 8-byte reads of the transposed page at keys 16 t + 4 h and
-// 16 t + 8 + 4 h.  So the probabilities never leave the registers.  The two lanes of a query
-// share its running maximum (one exchange a page) and keep separate sums.  The output tile has
-// lane (d column n, half h) hold queries 8 i + 4 h + r, so factors per query (the rescaling
-// when a maximum moves, the final 1 / sum) pass through 32 floats of LDS a wave.  Softmax
-// state is float32 (in units of log2); probabilities are rounded to bfloat16 for the value
-// product (the reference's prefill kernel does the same,
-// operators/src/cuda/kernels/flash_attn_prefill.cu:240).
+// in the same order.  They do, out of two transposing reads (ds_read_b64_tr_b16: in each 16
+// lanes, lane 4 q + e receives element e of the four 8-byte pieces that lanes q, q + 4, q + 8,
+// q + 12 point at): lane s of 16 points at key 4 h + s / 4 of the step (plus 8 for the second
+// read) and at d columns 16 (l / 16 % 2) + 4 (s % 4) .. + 3 of the 32-wide block.  So the
+// values need no transposition on their way into LDS and the probabilities never leave the
+// registers.  The two lanes of a query share its running maximum (one exchange a page) and
+// keep separate sums.  The output tile has lane (d column n, half h) hold queries
+// 8 i + 4 h + r, so factors per query (the rescaling when a maximum moves, the final 1 / sum)
+// pass through 32 floats of LDS a wave.  Softmax state is float32 (in units of log2);
+// probabilities are rounded to bfloat16 for the value product (the reference's prefill kernel
+// does the same, operators/src/cuda/kernels/flash_attn_prefill.cu:240).
 //
-// Keys lie in LDS as stored, with the 16-byte chunks of a row exchanged among themselves
-// (chunk ^ key % 16, for 64-wide heads chunk ^ (key / 2) % 8) so that the 16 rows a quarter
-// of a wave reads touch every bank once; values lie transposed ([d][key]).
+// Exchange of pieces.  Keys: the 16-byte chunks of a row, chunk ^ key % 16 (64-wide heads:
+// chunk ^ (key / 2) % 8), so that the 16 rows a quarter of a wave reads touch every bank once.
+// Values: the 32-byte pieces of a row, piece ^ 2 (key % 4) (64-wide heads: piece ^ 2 (key / 2
+// % 2)): the eight pieces that half a wave's transposing read takes (four keys, two pieces)
+// then lie in eight different eighths of the banks.
 // Blocks are numbered so that the blocks of one kv head fall on one XCD (the hardware deals
 // consecutive workgroups round-robin to its 8 XCDs): that head's keys and values then stay
 // in that XCD's L2.
 constexpr int kPrefillWaves = 8;
 constexpr int kPrefillThreads = kPrefillWaves * EI_WAVE;
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef short ei_s16x4 __attribute__((ext_vector_type(4)));
+typedef short ei_s16x8 __attribute__((ext_vector_type(8)));
 constexpr int kWideRows = 32;      // query rows of a wave
 constexpr int kAhead = 3;          // LDS operand reads in flight before the product that needs the first
+constexpr int kPageBuffers = 3;
+// (log2) how far a row's maximum may rise above the reference point of its exponentials before
+// the sums so far are rescaled to a new one: up to there the probabilities are merely larger
+// than 1 (at most 2^8, which bfloat16 and the float32 sums hold as well as values below 1).
+// Once the first pages are past, a page hardly ever moves any of a wave's 32 rows that far,
+// where a plain running maximum moves one of them on most pages: the rescaling (64 products
+// a lane and a trip through LDS) was a quarter of a page's vector work.
+constexpr float kLazyRise = 8.f;
 
 template <int D, int HB, int KW>
 __global__ void __launch_bounds__(kPrefillThreads, 2)
@@ -422,25 +448,25 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
                          int pair) {
   constexpr int SJ = D / 16;             // 16-wide steps over d for the scores
   constexpr int DB = D / 32;             // 32-wide output blocks over d
-  constexpr int VS = EI_PAGE + 4;        // LDS stride of a transposed value row (34 dwords)
-  constexpr int CI = D / 32;             // 16-byte chunks per thread per page
-  constexpr int CHUNKS = D / 8;          // 16-byte chunks of a key row
-  constexpr int KBUF = EI_PAGE * D, VBUF = D * VS;    // elements of one page buffer
+  constexpr int CHUNKS = D / 8;          // 16-byte chunks of a row
+  constexpr int PBUF = EI_PAGE * D;      // elements of one page of keys or of values
   constexpr int NG = kPrefillWaves / (HB * KW);       // groups of 32 rows in a block
   constexpr int KBL = 2 / KW;            // blocks of 32 keys of a page that a wave takes
+  // a page of keys and one of values are 2 * PBUF * 2 bytes, a wave load a kilobyte
+  constexpr int LOADS = 2 * PBUF * 2 / 1024 / kPrefillWaves;   // wave loads per wave and page
+  constexpr int ROWS_A_LOAD = 1024 / (2 * D);                  // rows a wave load covers
   static_assert(KW == 1 || KW == 2, "a page's keys go to one wave or to two");
   static_assert(NG >= 1, "eight waves: heads x row groups x key ways");
-  // two pages of keys and of (transposed) values alternate, so that a page costs one barrier
-  __shared__ __attribute__((aligned(16))) bf16_t page_lds[2 * KBUF + 2 * VBUF];
-  bf16_t* const k_lds = page_lds;
-  bf16_t* const v_lds = page_lds + 2 * KBUF;
+  static_assert(LOADS >= 2 && LOADS % 2 == 0, "a wave fetches as much of the keys as of the values");
+  // buffer b: keys at b * 2 * PBUF, values PBUF further
+  __shared__ __attribute__((aligned(1024))) bf16_t page_lds[kPageBuffers * 2 * PBUF];
   __shared__ __attribute__((aligned(16))) float factor_lds[kPrefillWaves][kWideRows];
   // (KW = 2) what the second wave of a (head, rows) pair hands to the first at the end: its
   // running maximum and sum per row here, its output tile in the page buffers
   __shared__ float handed_lds[KW == 2 ? kPrefillWaves / 2 : 1][2][kWideRows];
   __shared__ __attribute__((aligned(16))) float other_lds[KW == 2 ? kPrefillWaves : 1][kWideRows];
   static_assert(KW == 1 || (kPrefillWaves / 2) * (D / 32) * 16 * EI_WAVE * sizeof(float) <=
-                               sizeof(bf16_t) * (2 * KBUF + 2 * VBUF),
+                               sizeof(bf16_t) * kPageBuffers * 2 * PBUF,
                 "the handed-over output tiles fit the page buffers");
 
   const int G = nq / nkv;
@@ -469,27 +495,42 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
   const int n32 = lane & 31, half = lane >> 5;
   const int hw = wave % HB, pw = (wave / HB) % NG, kw = wave / (HB * NG);
   const int head = g * G + hb * HB + hw;
-  // a key row's chunk `chunk` lies at this place of the row
-  auto place = [](int key, int chunk) {
+  // where chunk `chunk` of key row `key` lies in the row, and the same for a row of values
+  auto k_place = [](int key, int chunk) {
     return CHUNKS == 16 ? (chunk ^ (key & 15)) : (chunk ^ ((key >> 1) & 7));
+  };
+  auto v_place = [](int key, int chunk) {
+    const int piece = chunk >> 1;
+    const int moved = D == 128 ? (piece ^ (2 * (key & 3))) : (piece ^ (2 * ((key >> 1) & 1)));
+    return 2 * moved + (chunk & 1);
   };
   // Everything a lane needs to find its operands in a page buffer is worked out once: the
   // places of its key chunks (they differ from step to step by the exchange of chunks; key
-  // blocks and buffers add constants), the place of its value words, and where its share of
-  // the next page goes.
-  int k_read[SJ];                        // (element offsets into the page buffers)
+  // blocks and buffers add constants) and of the value pieces its transposing reads point at.
+  int k_read[SJ];                        // (element offsets into a page of keys)
 #pragma unroll
-  for (int sj = 0; sj < SJ; ++sj) k_read[sj] = n32 * D + place(n32, 2 * sj + half) * 8;
-  const int v_read = n32 * VS + 4 * half;
-  // waves 0..3 move the page's keys, waves 4..7 its values: four lanes a row, chunks
-  // ld_dc + 4 i of it.  (With eight lanes a row the 16-bit stores of the values' transposition
-  // met every bank twice: rows 32 apart lie 16 banks apart four times over.)
-  const bool moves_values = t >= kPrefillThreads / 2;
-  const int ld_key = (t & (kPrefillThreads / 2 - 1)) >> 2, ld_dc = t & 3;
-  int k_write[CI];
+  for (int sj = 0; sj < SJ; ++sj) k_read[sj] = n32 * D + k_place(n32, 2 * sj + half) * 8;
+  int v_read[DB];                        // (element offsets into a page of values)
+  {
+    const int s16 = lane & 15, vkey = 4 * half + (s16 >> 2);
 #pragma unroll
-  for (int i = 0; i < CI; ++i) k_write[i] = ld_key * D + place(ld_key, ld_dc + 4 * i) * 8;
-  const int v_write = ld_dc * 8 * VS + ld_key;
+    for (int db = 0; db < DB; ++db)
+      v_read[db] = vkey * D + v_place(vkey, 2 * (2 * db + ((lane >> 4) & 1))) * 8 + 4 * (s16 & 3);
+  }
+  // The wave's loads of a page: load i < LOADS / 2 brings kilobyte wave + 8 i of the keys, the
+  // others the same of the values.  Lane l's 16 bytes land at place l % CHUNKS of row
+  // l / CHUNKS of that kilobyte; it fetches the chunk of the row that belongs there (both
+  // exchanges are their own inverses).
+  int fetch_from[LOADS];                 // element offsets into the page in global memory
+  int fetch_row[LOADS / 2];              // (values) the row of the page that the lane's piece belongs to
+#pragma unroll
+  for (int i = 0; i < LOADS; ++i) {
+    const int part = i % (LOADS / 2);
+    const int row = (wave + kPrefillWaves * part) * ROWS_A_LOAD + lane / CHUNKS;
+    const int at = lane % CHUNKS;
+    fetch_from[i] = row * D + (i < LOADS / 2 ? k_place(row, at) : v_place(row, at)) * 8;
+    if (i >= LOADS / 2) fetch_row[part] = row;
+  }
 
   for (int pass = 0; pass <= pair; ++pass) {
   const int item = pass == 0 ? unit : n_items - 1 - unit;
@@ -534,61 +575,61 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 #pragma unroll
     for (int e = 0; e < 16; ++e) o_acc[db][e] = 0.f;
 
-  uint4 stage[CI];
-  auto lookup = [&](int page_index) __attribute__((always_inline)) {
-    return page_index <= hi_page
-               ? page_table[static_cast<size_t>(seq) * table_width + page_index] : -1;
+  // Request page `page_index` of the sequence into buffer `buf` (nothing past the last page).
+  // A page that the window has given back (none of its keys is visible to any row: it only
+  // lies in the walk) is cleared instead, by plain stores.
+  auto fetch_page = [&](int page_index, int buf) __attribute__((always_inline)) {
+    if (page_index > hi_page) return;
+    const int phys = page_table[static_cast<size_t>(seq) * table_width + page_index];
+    bf16_t* const to = page_lds + buf * 2 * PBUF;
+    if (phys < 0) {
+#pragma unroll
+      for (int i = 0; i < LOADS; ++i)
+        *reinterpret_cast<uint4*>(to + (i / (LOADS / 2)) * PBUF +
+                                  (wave + kPrefillWaves * (i % (LOADS / 2))) * 512 + lane * 8) =
+            uint4{0u, 0u, 0u, 0u};
+      // (the waits below count a page's loads: with none for this page, everything requested
+      // before must have arrived here)
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+      return;
+    }
+    const size_t base = (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+      const bf16_t* const from = (i < LOADS / 2 ? k_pages : v_pages) + base + fetch_from[i];
+      __builtin_amdgcn_global_load_lds(
+          (const __attribute__((address_space(1))) void*)from,
+          (__attribute__((address_space(3))) void*)(to + (i / (LOADS / 2)) * PBUF +
+                                                    (wave + kPrefillWaves * (i % (LOADS / 2))) * 512),
+          16, 0, 0);
+    }
   };
-  auto load_page = [&](int page_index, int phys) __attribute__((always_inline)) {
-    if (phys < 0) {                       // released by the window: every key is masked
+  // The wave's loads of page `page_index` have arrived (all but the `younger` loads it has
+  // requested since): if it is the sequence's last page, the value rows beyond the item's
+  // last position are cleared, each piece by the lane that fetched it.
+  auto page_arrived = [&](int page_index, int buf, auto younger_tag) __attribute__((always_inline)) {
+    constexpr int younger = decltype(younger_tag)::value;
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (younger & 15) | ((younger >> 4) << 14));
+    if (page_index == hi_page) {
+      bf16_t* const to = page_lds + buf * 2 * PBUF + PBUF;
 #pragma unroll
-      for (int i = 0; i < CI; ++i) stage[i] = uint4{0u, 0u, 0u, 0u};
-      return;
+      for (int part = 0; part < LOADS / 2; ++part)
+        if (page_index * EI_PAGE + fetch_row[part] > last_pos)
+          *reinterpret_cast<uint4*>(to + (wave + kPrefillWaves * part) * 512 + lane * 8) =
+              uint4{0u, 0u, 0u, 0u};
     }
-    const bf16_t* const src =
-        (moves_values ? v_pages : k_pages) +
-        ((static_cast<size_t>(phys) * nkv + g) * EI_PAGE + ld_key) * D + ld_dc * 8;
-    if (page_index < hi_page) {           // a whole page (the same for every lane)
-#pragma unroll
-      for (int i = 0; i < CI; ++i) stage[i] = *reinterpret_cast<const uint4*>(src + 32 * i);
-      return;
-    }
-    const bool live = page_index * EI_PAGE + ld_key <= last_pos;   // later slots: stale bytes
-#pragma unroll
-    for (int i = 0; i < CI; ++i)
-      stage[i] = live ? *reinterpret_cast<const uint4*>(src + 32 * i) : uint4{0u, 0u, 0u, 0u};
-  };
-  // Values go to LDS transposed ([d][key]): a lane holds 8 values of one key and stores each
-  // as 16 bits at its d row (the row offsets are constants of the instruction, the upper
-  // halves are stored from where they are), which costs no vector arithmetic at all; an
-  // exchange of halves between lanes and dword stores was 50 vector instructions a page more.
-  auto store_page = [&](auto buf_tag) __attribute__((always_inline)) {
-    constexpr int buf = decltype(buf_tag)::value;
-    if (!moves_values) {
-#pragma unroll
-      for (int i = 0; i < CI; ++i)
-        *reinterpret_cast<uint4*>(&k_lds[k_write[i] + buf * KBUF]) = stage[i];
-      return;
-    }
-#pragma unroll
-    for (int i = 0; i < CI; ++i) {
-      const uint32_t w[4] = {stage[i].x, stage[i].y, stage[i].z, stage[i].w};
-      bf16_t* const to = &v_lds[v_write + buf * VBUF + 4 * i * 8 * VS];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        to[(2 * e) * VS] = static_cast<bf16_t>(w[e] & 0xffffu);
-        to[(2 * e + 1) * VS] = static_cast<bf16_t>(w[e] >> 16);
-      }
-    }
+    __syncthreads();
+    __builtin_amdgcn_sched_barrier(0);
   };
 
-  // The scores of one page from LDS buffer `buf`, their softmax into `p_reg` (A operands of P
+  // The scores of one page from buffer `buf`, their softmax into `p_reg` (A operands of P
   // for the four 16-key steps), and the rescaling of the output so far.  MASKED: some key of
   // the page is hidden from some row of the wave (all but the last one or two pages of a
   // causal prompt need no mask).
   bf16x8 p_reg[2 * KBL];
-  auto scores = [&](const int key_base, auto buf_tag, const bool MASKED) __attribute__((always_inline)) {
-    constexpr int buf = decltype(buf_tag)::value;
+  auto scores = [&](const int key_base, const int buf, const bool MASKED) __attribute__((always_inline)) {
+    const bf16_t* const k_lds = page_lds + buf * 2 * PBUF;
     f32x16 s[KBL];
 #pragma unroll
     for (int kb = 0; kb < KBL; ++kb)
@@ -599,7 +640,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
 #pragma unroll
       for (int kb = 0; kb < KBL; ++kb) {
         const bf16x8 kf = *reinterpret_cast<const bf16x8*>(
-            &k_lds[k_read[sj] + buf * KBUF + (kw * KBL + kb) * 32 * D]);
+            &k_lds[k_read[sj] + (kw * KBL + kb) * 32 * D]);
         s[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf, q_reg[sj], s[kb], 0, 0, 0);
       }
     // instruction order: the operand reads from LDS run kAhead products ahead of the products
@@ -635,9 +676,12 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
                                                            __float_as_uint(tile_max), false, false);
       tile_max = fmaxf(__uint_as_float(both.x), __uint_as_float(both.y));
     }
-    // running maximum in units of log2 (raw score * scale * log2 e; the scale is positive);
-    // a row with no visible key yet keeps the lowest value, not -inf, so that no NaN arises
-    const float m_new = fmaxf(m_run, tile_max * scale_log2);
+    // The reference point of the row's exponentials, in units of log2 (raw score * scale *
+    // log2 e; the scale is positive): it follows the maximum only when that has risen by more
+    // than kLazyRise.  A row with no visible key yet keeps the lowest value, not -inf, so that
+    // no NaN arises.
+    const float m_tile = tile_max * scale_log2;
+    const float m_new = m_tile > m_run + kLazyRise ? m_tile : m_run;
     const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
     float tile_sum = 0.f;
 #pragma unroll
@@ -653,7 +697,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
         }
     l_run = l_run * alpha + tile_sum;
     m_run = m_new;
-    if (__any(alpha != 1.f)) {            // the maximum of some row of this wave has moved
+    if (__any(alpha != 1.f)) {            // the reference point of some row of this wave has moved
       if (half == 0) factor_lds[wave][n32] = alpha;
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
@@ -674,25 +718,26 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     }
   };
   // output += P V for the page whose probabilities are in `p_reg`, values from buffer `buf`
-  auto values = [&](auto buf_tag) __attribute__((always_inline)) {
-    constexpr int buf = decltype(buf_tag)::value;
+  auto values = [&](const int buf) __attribute__((always_inline)) {
+    typedef __attribute__((address_space(3))) ei_s16x4 lds_s16x4;
+    const bf16_t* const v_lds = page_lds + buf * 2 * PBUF + PBUF;
 #pragma unroll
     for (int st = 0; st < 2 * KBL; ++st) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
-        const bf16_t* vrow = &v_lds[v_read + buf * VBUF + db * 32 * VS + (kw * 2 * KBL + st) * 16];
-        const uint2 lo = *reinterpret_cast<const uint2*>(vrow);
-        const uint2 hi = *reinterpret_cast<const uint2*>(vrow + 8);
-        uint4 both = uint4{lo.x, lo.y, hi.x, hi.y};
-        const bf16x8 vf = *reinterpret_cast<bf16x8*>(&both);
-        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(p_reg[st], vf, o_acc[db], 0, 0, 0);
+        const bf16_t* vrow = &v_lds[v_read[db] + (kw * 2 * KBL + st) * 16 * D];
+        const ei_s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow));
+        const ei_s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(vrow + 8 * D));
+        const ei_s16x8 both = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o_acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+            p_reg[st], __builtin_bit_cast(bf16x8, both), o_acc[db], 0, 0, 0);
       }
     }
-    __builtin_amdgcn_sched_group_barrier(0x100, kAhead, 0);      // as for the scores
+    __builtin_amdgcn_sched_group_barrier(0x100, 2 * kAhead, 0);      // as for the scores
 #pragma unroll
     for (int n = 0; n < 2 * KBL * DB; ++n) {
       __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
     }
   };
   // whether this wave has anything to do with a page: one that lies wholly after the wave's
@@ -703,44 +748,33 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_p
     return wave_has_rows && key_lo <= wave_last_pos &&
            (window <= 0 || !wave_rows_valid || key_hi > wave_min_pos - window);
   };
-  auto scores_of = [&](const int page, auto buf_tag) __attribute__((always_inline)) {
+  auto scores_of = [&](const int page, const int buf) __attribute__((always_inline)) {
     const int key_base = page * EI_PAGE;
     const int key_lo = key_base + kw * KBL * 32, key_hi = key_lo + KBL * 32 - 1;
     const bool no_mask = wave_rows_valid && key_hi <= wave_min_pos &&
                          (window <= 0 || key_lo > wave_max_pos - window);
-    scores(key_base, buf_tag, !no_mask);
+    scores(key_base, buf, !no_mask);
   };
-  // Page p is multiplied from buffer p & 1 while page p + 1 (fetched a page ago) goes from
-  // registers into the other buffer and page p + 2 is requested; the barrier at the end of a
-  // page says both that the other buffer is complete and that this one is free.
-  int phys_next;
-  auto one_page = [&](const int page, auto buf_tag) __attribute__((always_inline)) {
-    constexpr int buf = decltype(buf_tag)::value;
+  using Both = std::integral_constant<int, LOADS>;
+  using None = std::integral_constant<int, 0>;
+  fetch_page(lo_page, 0);
+  fetch_page(lo_page + 1, 1);
+  if (lo_page + 1 <= hi_page) page_arrived(lo_page, 0, Both{});
+  else page_arrived(lo_page, 0, None{});
+  int buf = 0;
+  for (int page = lo_page; page <= hi_page; ++page) {
+    const int next = buf == kPageBuffers - 1 ? 0 : buf + 1;
+    fetch_page(page + 2, next == kPageBuffers - 1 ? 0 : next + 1);
+    __builtin_amdgcn_sched_barrier(0);
     if (page_seen(page)) {
-      scores_of(page, buf_tag);
-      values(buf_tag);
+      scores_of(page, buf);
+      values(buf);
     }
     if (page < hi_page) {
-      store_page(std::integral_constant<int, 1 - buf>{});
-      load_page(page + 2, phys_next);
-      phys_next = lookup(page + 3);
-      __syncthreads();
+      if (page + 2 <= hi_page) page_arrived(page + 1, next, Both{});
+      else page_arrived(page + 1, next, None{});
     }
-  };
-  load_page(lo_page, lookup(lo_page));
-  if (lo_page & 1) store_page(std::integral_constant<int, 1>{});
-  else store_page(std::integral_constant<int, 0>{});
-  load_page(lo_page + 1, lookup(lo_page + 1));    // zeros past the last page
-  phys_next = lookup(lo_page + 2);
-  __syncthreads();
-  int page = lo_page;
-  if (page & 1) {
-    one_page(page, std::integral_constant<int, 1>{});
-    ++page;
-  }
-  for (; page <= hi_page; page += 2) {
-    one_page(page, std::integral_constant<int, 0>{});
-    if (page + 1 <= hi_page) one_page(page + 1, std::integral_constant<int, 1>{});
+    buf = next;
   }
 
   // 1 / sum per query through LDS; lane (d column n32, half) holds O[query 8 i + 4 half + r]
