@@ -18,7 +18,8 @@ steps timed as steps, its prompt step) and decode at batch 1 and 16 and the pref
 32B shape (`--without-32b` leaves those out).  `points` is flat: beside every rate `<name>`
 stand `<name>_ms` (a step), `<name>_GB` (what the step has to read, or `_TFLOP`: what it has
 to multiply), `<name>_frac` (of the published peak) and `<name>_frac_measured` (of what the
-chip at hand gives).
+chip at hand gives).  `decode_b8_launches` and `decode_b8_launch_floor_ms`: the kernel launches
+of a decode step, and what a graph of as many launches of a kernel that does nothing takes.
 Synthetic token ids, seeded random weights N(0, 0.02).  Peaks are the MI355X's published
 ones: HBM 8 TB/s, dense bf16 MFMA 2.5 PFLOP/s; `measured_peaks` (and `--peaks` alone) say what
 a plain read kernel and a loop of matrix-core products reach on the GPU at hand, and the
@@ -225,6 +226,37 @@ def measure_peaks():
             "mfma_bf16_TFLOPs": round(flops / mfma_s / 1e12, 1)}
 
 
+def measure_launch_floor(model, cfg, batch, replays=50):
+    """(kernel launches of one decode step, ms a replay of a graph of as many launches of a
+    kernel that does nothing): what the chain of dependent launches alone costs, the floor
+    under a step of this design whatever its kernels do."""
+    import torch
+    import edge_infer_amd as ei
+    from edge_infer_amd.csrc import lib
+    session = ei.Session(model, max_tokens=batch * 1024, max_seqs=batch, max_seq_tokens=1024,
+                         graphs=False)
+    prompts = synthetic_prompts(cfg, batch, 64, seed=9)
+    slots = [session.begin() for _ in range(batch)]
+    session.step([(s, p, [63]) for s, p in zip(slots, prompts)], copy=False)
+    before = lib.launches
+    session.step([(s, [1], [0]) for s in slots], copy=False)
+    count = lib.launches - before
+    del session
+    lib.empty_launches(4)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        lib.empty_launches(count)
+    for _ in range(3):
+        graph.replay()
+    torch.cuda.synchronize()
+    started = time.perf_counter()
+    for _ in range(replays):
+        graph.replay()
+    torch.cuda.synchronize()
+    return count, 1000.0 * (time.perf_counter() - started) / replays
+
+
 def data_bytes_of(gib):
     return gib * 1024 ** 3
 
@@ -382,6 +414,10 @@ def main():
                                    graphs=False)
         decode_point(points, f"decode_b{args.batch}_eager", cfg, args.batch, ms, args.batch * at,
                      itemsize, peaks)
+        # what the step's chain of launches costs with kernels that do nothing
+        count, floor_ms = measure_launch_floor(model, cfg, args.batch)
+        points[f"decode_b{args.batch}_launches"] = count
+        points[f"decode_b{args.batch}_launch_floor_ms"] = round(floor_ms, 4)
     if not args.skip_points and args.shape == "8b":
         del model
         torch.cuda.empty_cache()

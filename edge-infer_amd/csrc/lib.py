@@ -86,6 +86,7 @@ _SIGNATURES = {
     "peaks": {
         "ei_stream_read": [c_void_p, c_longlong, c_int, c_void_p, c_void_p],
         "ei_mfma_loop": [c_int, c_int, c_int, c_void_p, c_void_p],
+        "ei_empty_launches": [c_int, c_int, c_void_p],
     },
 }
 
@@ -124,7 +125,12 @@ def prepare(names) -> None:
     build.build_libraries([name for name in names if name not in _loaded])
 
 
+launches = 0        # calls of kernel entry points so far (most launch one kernel, a few two)
+
+
 def _check(lib, status: int, what: str) -> None:
+    global launches
+    launches += 1
     if status != 0:
         message = lib.ei_last_error().decode(errors="replace")
         raise KernelError(f"{what}: {message} (status {status})")
@@ -683,3 +689,10 @@ def mfma_loop(iters: int, blocks: int, sink: torch.Tensor, wide: bool = False) -
     status = lib.ei_mfma_loop(int(iters), int(blocks), int(wide),
                               _gpu(sink, "sink", torch.float32), _stream())
     _check(lib, status, "mfma_loop")
+
+
+def empty_launches(count: int, blocks: int = 256) -> None:
+    """`count` launches of a kernel that does nothing (`blocks` blocks of one wave), one after
+    the other on the current stream: the floor under a chain of that many dependent kernels."""
+    lib = library("peaks")
+    _check(lib, lib.ei_empty_launches(int(count), int(blocks), _stream()), "empty_launches")

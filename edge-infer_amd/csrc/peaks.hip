@@ -1,5 +1,6 @@
-// Two yardsticks for the measurements: how fast this GPU streams memory through a plain read
-// kernel, and how fast its matrix cores multiply when nothing else is asked of them.  The
+// Yardsticks for the measurements: how fast this GPU streams memory through a plain read
+// kernel, how fast its matrix cores multiply when nothing else is asked of them, and what a
+// chain of launches costs when the kernels do nothing.  The
 // published peaks (8 TB/s, 2.5 PFLOP/s dense bfloat16) are what the figures are priced
 // against; these kernels say how much of them any kernel can get on the machine at hand.
 #include "common.h"
@@ -85,7 +86,20 @@ mfma_loop_wide_kernel(int iters, float* __restrict__ sink) {
   if (total == 12345.678f) sink[0] = total;
 }
 
+// A kernel that does nothing: what a launch costs when nothing is computed.
+__global__ void empty_kernel(int) {}
+
 }  // namespace
+
+// `count` launches of a kernel that does nothing, `blocks` blocks of one wave each, one after
+// the other on `stream`: captured in a graph they are the floor under any chain of that many
+// dependent kernels.
+extern "C" int ei_empty_launches(int count, int blocks, hipStream_t stream) {
+  EI_REQUIRE(count >= 1 && count <= 1 << 20 && blocks >= 1 && blocks <= 1 << 20,
+             "empty_launches: bad sizes");
+  for (int i = 0; i < count; ++i) empty_kernel<<<blocks, EI_WAVE, 0, stream>>>(i);
+  EI_LAUNCH_CHECK();
+}
 
 // Reads `bytes` (a multiple of 16) from `data` once, with `blocks` blocks of 256 threads.
 extern "C" int ei_stream_read(const void* data, long long bytes, int blocks, void* sink,
