@@ -29,11 +29,17 @@ MAX_GRAPHS = 24         # captured decode steps a session keeps; the one unused 
 
 def batch_bucket(live: int) -> int:
     """The fixed batch size a decode step of `live` sequences is padded to when it is
-    captured: powers of two up to 64, then multiples of 32."""
-    bucket = 1
-    while bucket < live and bucket < 64:
-        bucket *= 2
-    return bucket if bucket >= live else (live + 31) // 32 * 32
+    captured: powers of two up to 16, multiples of 8 up to 64, then multiples of 32.  (A
+    padding row costs what a live one costs: 48 sequences in a step for 64 took 4.63 ms for
+    the 8B shape where the step for 48 takes 4.46.)"""
+    if live <= 16:
+        bucket = 1
+        while bucket < live:
+            bucket *= 2
+        return bucket
+    if live <= 64:
+        return (live + 7) // 8 * 8
+    return (live + 31) // 32 * 32
 
 
 def context_bound(context: int, capacity: int) -> int:

@@ -137,18 +137,20 @@ class Attention:
 
     def prefill_key_ways(self, counts) -> int:
         """1 or 2: how many waves share the keys of a page for the same rows in the prompt
-        step whose sequences bring `counts` tokens.  The matrix-core kernel pairs a long item
-        with a short one per block once there are 512 blocks, which loads every block alike;
-        a step with fewer blocks than that (one prompt of 2,048 tokens of the 8B shape has
-        256, whose walks are 1 to 32 pages long) takes items half as long, and with them
-        twice the blocks."""
+        step whose sequences bring `counts` tokens.  A step that gives every compute unit
+        about one block (one prompt of 2,048 tokens of the 8B shape: 256, whose walks are 1 to
+        32 pages long) takes items half as long, and with them twice the blocks, which the
+        kernel then pairs, a long one with a short one; with more blocks than that the
+        hardware balances them, and a wave that takes every key of a page for its rows does
+        less beside its products (measured, one prompt of the 8B shape: 2,048 tokens 60
+        against 71 us, 3,072 tokens 147 against 105)."""
         if not self.matrix_cores or self.positions_per_item(2) == 0:
             return 1
         size = self.positions_per_item(1)
         heads = lib.attention_prefill_mfma_heads(self.group)
         items = sum((count + size - 1) // size for count in counts)
         blocks = items * (self.group // heads) * self.spec.n_kv_heads
-        return 2 if blocks < 2 * self.compute_units else 1
+        return 2 if 4 * blocks <= 5 * self.compute_units else 1
 
     @property
     def plan_key(self):
