@@ -715,8 +715,9 @@ def test_sample_refuses_bad_policies(lib):
 
 
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64, 65, 130, 256])
-@pytest.mark.parametrize("N,K", [(381, 96), (200, 200), (96, 256), (4096, 1024), (1000, 1384)])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 64, 65, 128, 129, 130, 256])
+@pytest.mark.parametrize("N,K", [(381, 96), (200, 200), (96, 256), (4096, 1024), (1000, 1384),
+                                 (16400, 264)])
 def test_gemm_bf16_skinny(lib, M, N, K):
     """The weight-streaming product for few rows: every slice count it may choose, widths
     that are no multiple of the tile, the same row alone or among others, and more than 64
