@@ -60,6 +60,41 @@ template <> struct Vec4<bf16_t> {
   }
 };
 
+// P consecutive elements (4 or 8) of type T as floats; eight bfloat16 travel as one 16-byte
+// access.
+template <typename T, int P> struct VecN;
+template <typename T> struct VecN<T, 4> : Vec4<T> {};
+template <> struct VecN<float, 8> {
+  static __device__ __forceinline__ void load(const float* p, float (&v)[8]) {
+    const float4 x = *reinterpret_cast<const float4*>(p), y = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = x.x; v[1] = x.y; v[2] = x.z; v[3] = x.w;
+    v[4] = y.x; v[5] = y.y; v[6] = y.z; v[7] = y.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[8]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    *reinterpret_cast<float4*>(p + 4) = make_float4(v[4], v[5], v[6], v[7]);
+  }
+};
+template <> struct VecN<bf16_t, 8> {
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 x = *reinterpret_cast<const uint4*>(p);
+    const uint32_t u[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __uint_as_float(u[i] << 16);
+      v[2 * i + 1] = __uint_as_float(u[i] & 0xffff0000u);
+    }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    uint32_t u[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      u[i] = static_cast<uint32_t>(f32_to_bf16(v[2 * i])) |
+             (static_cast<uint32_t>(f32_to_bf16(v[2 * i + 1])) << 16);
+    *reinterpret_cast<uint4*>(p) = uint4{u[0], u[1], u[2], u[3]};
+  }
+};
+
 // x / (1 + e^-x).  For a float32 result the library's exponential and a true division;
 // for a bfloat16 result (8 bits of mantissa) the hardware's exp2 and reciprocal, both good
 // to about one unit in the 23rd bit, which the rounding to bfloat16 swallows.

@@ -117,36 +117,45 @@ __global__ void qk_norm_rope_store_kernel(
   }
 }
 
-// The same for head sizes (and rotated widths) that are a multiple of 8: G lanes (a power of
-// two) share a head, each lane takes 4 neighbouring pairs with one 8- or 16-byte access per
-// half, so a wave covers 64 / G heads.
-template <typename TI, typename TO, int G>
-__global__ void qk_norm_rope_store_vec_kernel(
-    const TI* __restrict__ qkv, int nsplit, size_t split_stride,
+// The same for head sizes (and rotated widths) that are a multiple of 2 P: G lanes (a power of
+// two) share a head, each lane takes P (4 or 8) neighbouring pairs with one or two 16-byte
+// accesses (one of 8 bytes for 4 bfloat16) per half, so a wave covers 64 / G heads.
+template <typename TI, typename TO, int G, int P>
+__device__ __forceinline__ void qk_norm_rope_store_item(
+    long long item, int sub, const TI* __restrict__ qkv, int nsplit, size_t split_stride,
     const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
     const float* __restrict__ rope_table, const int32_t* __restrict__ row_pos,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
     TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
     int N, int nq, int nkv, int D, int R, int write_cache) {
-  using ei::Vec4;
+  using ei::VecN;
   const int heads = nq + 2 * nkv;
-  const long long item = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) / G;
-  const int sub = threadIdx.x % G;
-  if (item >= static_cast<long long>(N) * heads) return;       // the same for all lanes of a group
   const int row = static_cast<int>(item / heads), head = static_cast<int>(item % heads);
-  const int seq = row_seq[row];
-  if (seq < 0) return;  // padding row
   const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
   if (!is_q && !write_cache) return;
+  // The sequence and the position are asked for first and the head's elements right after,
+  // before either is needed: what depends on them (the page, the angles) is then looked up
+  // while the elements are on their way.  (A padding row costs its loads.)
+  const int seq = row_seq[row];
   const int pos = row_pos[row];
   const int half = D / 2, rhalf = R / 2;
-  const int pair0 = sub * 4;                                   // the lane's first pair
+  const int pair0 = sub * P;                                   // the lane's first pair
   const bool active = pair0 < half;
-  const bool turned = pair0 < rhalf;                           // its four pairs are rotated ones
+  const bool turned = pair0 < rhalf;                           // its pairs are rotated ones
   const int i0 = turned ? pair0 : pair0 + rhalf;               // their first elements
   const int i2 = turned ? pair0 + rhalf : pair0 + half;        // and their second ones
   const size_t width = static_cast<size_t>(heads) * D;
   const TI* src = qkv + static_cast<size_t>(row) * width + static_cast<size_t>(head) * D;
+  float first_a[4][P], first_b[4][P];                          // the first four slices
+  if (active) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (u < nsplit) {
+        VecN<TI, P>::load(src + u * split_stride + i0, first_a[u]);
+        VecN<TI, P>::load(src + u * split_stride + i2, first_b[u]);
+      }
+  }
+  if (seq < 0) return;  // padding row
 
   TO* dst;
   bool stored = true;
@@ -162,51 +171,63 @@ __global__ void qk_norm_rope_store_vec_kernel(
   const float* norm_w = is_q ? q_norm_w : (is_k ? k_norm_w : nullptr);
   const bool rotate = rope_table != nullptr && (is_q || is_k);
 
-  float x[4] = {0.f, 0.f, 0.f, 0.f}, y[4] = {0.f, 0.f, 0.f, 0.f};
-  float wx[4] = {1.f, 1.f, 1.f, 1.f}, wy[4] = {1.f, 1.f, 1.f, 1.f};
-  float cs[4] = {1.f, 1.f, 1.f, 1.f}, sn[4] = {0.f, 0.f, 0.f, 0.f};
+  float x[P], y[P], wx[P], wy[P], cs[P], sn[P];
+#pragma unroll
+  for (int i = 0; i < P; ++i) {
+    x[i] = y[i] = sn[i] = 0.f;
+    wx[i] = wy[i] = cs[i] = 1.f;
+  }
   if (active) {
-    for (int s0 = 0; s0 < nsplit; s0 += 4) {       // slices in slice order, four per trip
-      float a[4][4], b[4][4];
+    if (norm_w) {
+      VecN<float, P>::load(norm_w + i0, wx);
+      VecN<float, P>::load(norm_w + i2, wy);
+    }
+    if (rotate && turned) {
+      const float* trig = rope_table + static_cast<size_t>(pos) * R + pair0;
+      VecN<float, P>::load(trig, cs);
+      VecN<float, P>::load(trig + rhalf, sn);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (u < nsplit) {
+#pragma unroll
+        for (int i = 0; i < P; ++i) {
+          x[i] += first_a[u][i];
+          y[i] += first_b[u][i];
+        }
+      }
+    for (int s0 = 4; s0 < nsplit; s0 += 4) {       // further slices in slice order, four per trip
+      float a[4][P], b[4][P];
 #pragma unroll
       for (int u = 0; u < 4; ++u)
         if (s0 + u < nsplit) {
-          Vec4<TI>::load(src + (s0 + u) * split_stride + i0, a[u]);
-          Vec4<TI>::load(src + (s0 + u) * split_stride + i2, b[u]);
+          VecN<TI, P>::load(src + (s0 + u) * split_stride + i0, a[u]);
+          VecN<TI, P>::load(src + (s0 + u) * split_stride + i2, b[u]);
         }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
         if (s0 + u < nsplit) {
 #pragma unroll
-          for (int i = 0; i < 4; ++i) {
+          for (int i = 0; i < P; ++i) {
             x[i] += a[u][i];
             y[i] += b[u][i];
           }
         }
-    }
-    if (norm_w) {
-      Vec4<float>::load(norm_w + i0, wx);
-      Vec4<float>::load(norm_w + i2, wy);
-    }
-    if (rotate && turned) {
-      const float* trig = rope_table + static_cast<size_t>(pos) * R + pair0;
-      Vec4<float>::load(trig, cs);
-      Vec4<float>::load(trig + rhalf, sn);
     }
   }
   float inv = 1.f;
   if (norm_w) {
     float sum = 0.f;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) sum += x[i] * x[i] + y[i] * y[i];
+    for (int i = 0; i < P; ++i) sum += x[i] * x[i] + y[i] * y[i];
 #pragma unroll
     for (int offset = G / 2; offset > 0; offset >>= 1) sum += __shfl_xor(sum, offset, EI_WAVE);
     inv = rsqrtf(sum / static_cast<float>(D) + eps);
   }
   if (!active || !stored) return;
-  float ox[4], oy[4];
+  float ox[P], oy[P];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < P; ++i) {
     float a = x[i], b = y[i];
     if (norm_w) {
       a = (a * inv) * wx[i];
@@ -221,8 +242,24 @@ __global__ void qk_norm_rope_store_vec_kernel(
     ox[i] = a;
     oy[i] = b;
   }
-  Vec4<TO>::store(dst + i0, ox);
-  Vec4<TO>::store(dst + i2, oy);
+  VecN<TO, P>::store(dst + i0, ox);
+  VecN<TO, P>::store(dst + i2, oy);
+}
+
+template <typename TI, typename TO, int G, int P>
+__global__ void qk_norm_rope_store_vec_kernel(
+    const TI* __restrict__ qkv, int nsplit, size_t split_stride,
+    const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    const float* __restrict__ rope_table, const int32_t* __restrict__ row_pos,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ page_table, int table_width,
+    TO* __restrict__ q_out, TO* __restrict__ k_pages, TO* __restrict__ v_pages,
+    int N, int nq, int nkv, int D, int R, int write_cache) {
+  const long long item = (static_cast<long long>(blockIdx.x) * blockDim.x + threadIdx.x) / G;
+  const int sub = threadIdx.x % G;
+  if (item >= static_cast<long long>(N) * (nq + 2 * nkv)) return;   // the same for all lanes of a group
+  qk_norm_rope_store_item<TI, TO, G, P>(item, sub, qkv, nsplit, split_stride, q_norm_w, k_norm_w,
+                                        eps, rope_table, row_pos, row_seq, page_table, table_width,
+                                        q_out, k_pages, v_pages, N, nq, nkv, D, R, write_cache);
 }
 
 }  // namespace
@@ -250,38 +287,43 @@ extern "C" int ei_qk_norm_rope_store(
   const int heads = nq + 2 * nkv;
   const int threads = 256;
   const size_t ss = static_cast<size_t>(split_stride);
-  // vector kernel: 4 pairs a lane, G = lanes a head (the power of two at or above D/8)
+  // vector kernel: P pairs a lane (8 for bfloat16 in and out where the sizes allow, else 4),
+  // G = lanes a head (the power of two at or above D / 2P)
   const bool aligned = (reinterpret_cast<uintptr_t>(qkv) | reinterpret_cast<uintptr_t>(q_out) |
                         reinterpret_cast<uintptr_t>(k_pages) | reinterpret_cast<uintptr_t>(v_pages) |
                         reinterpret_cast<uintptr_t>(q_norm_w) | reinterpret_cast<uintptr_t>(k_norm_w) |
                         reinterpret_cast<uintptr_t>(rope_table)) % 16 == 0;
   if (D % 8 == 0 && R % 8 == 0 && ss % 4 == 0 && aligned) {
-    int G = 1;
-    while (G * 8 < D) G *= 2;
+    const bool wide = in_dtype == EI_BF16 && out_dtype == EI_BF16 && D % 16 == 0 && R % 16 == 0 &&
+                      ss % 8 == 0;
+    const int per_lane = wide ? 16 : 8;            // elements of a head a lane takes
+    int G = 2;
+    while (G * per_lane < D) G *= 2;
     const long long items = static_cast<long long>(N) * heads;
     const long long blocks = (items * G + threads - 1) / threads;
     EI_REQUIRE(blocks < (1ll << 31), "qk_norm_rope_store: too many rows");
-#define EI_ROPE_VEC(TI, TO, GG)                                                                   \
-  qk_norm_rope_store_vec_kernel<TI, TO, GG><<<static_cast<unsigned>(blocks), threads, 0, stream>>>( \
+#define EI_ROPE_VEC(TI, TO, GG, PP)                                                               \
+  qk_norm_rope_store_vec_kernel<TI, TO, GG, PP><<<static_cast<unsigned>(blocks), threads, 0, stream>>>( \
       static_cast<const TI*>(qkv), nsplit, ss, q_norm_w, k_norm_w, eps, rope_table, row_pos,      \
       row_seq, page_table, table_width, static_cast<TO*>(q_out), static_cast<TO*>(k_pages),       \
       static_cast<TO*>(v_pages), N, nq, nkv, D, R, write_cache)
-#define EI_ROPE_VEC_G(TI, TO)                                                                     \
+#define EI_ROPE_VEC_G(TI, TO, PP)                                                                 \
   do {                                                                                            \
-    if (G <= 2) EI_ROPE_VEC(TI, TO, 2);                                                           \
-    else if (G == 4) EI_ROPE_VEC(TI, TO, 4);                                                      \
-    else if (G == 8) EI_ROPE_VEC(TI, TO, 8);                                                      \
-    else if (G == 16) EI_ROPE_VEC(TI, TO, 16);                                                    \
-    else if (G == 32) EI_ROPE_VEC(TI, TO, 32);                                                    \
-    else EI_ROPE_VEC(TI, TO, 64);                                                                 \
+    if (G == 2) EI_ROPE_VEC(TI, TO, 2, PP);                                                       \
+    else if (G == 4) EI_ROPE_VEC(TI, TO, 4, PP);                                                  \
+    else if (G == 8) EI_ROPE_VEC(TI, TO, 8, PP);                                                  \
+    else if (G == 16) EI_ROPE_VEC(TI, TO, 16, PP);                                                \
+    else if (G == 32) EI_ROPE_VEC(TI, TO, 32, PP);                                                \
+    else EI_ROPE_VEC(TI, TO, 64, PP);                                                             \
   } while (0)
-    if (G <= 2) G = 2;
-    if (in_dtype == EI_F32 && out_dtype == EI_F32)
-      EI_ROPE_VEC_G(float, float);
+    if (wide)
+      EI_ROPE_VEC_G(bf16_t, bf16_t, 8);
+    else if (in_dtype == EI_F32 && out_dtype == EI_F32)
+      EI_ROPE_VEC_G(float, float, 4);
     else if (in_dtype == EI_F32 && out_dtype == EI_BF16)
-      EI_ROPE_VEC_G(float, bf16_t);
+      EI_ROPE_VEC_G(float, bf16_t, 4);
     else if (in_dtype == EI_BF16 && out_dtype == EI_BF16)
-      EI_ROPE_VEC_G(bf16_t, bf16_t);
+      EI_ROPE_VEC_G(bf16_t, bf16_t, 4);
     else
       EI_REQUIRE(false, "qk_norm_rope_store: unsupported dtype combination");
 #undef EI_ROPE_VEC_G
