@@ -81,19 +81,21 @@ def toy_skeleton_model_class():
     return ToySkeletonModel
 
 
-def toy_skeleton_oracle(cfg, weights, ids):
+def toy_skeleton_oracle(cfg, weights, ids, rope=plain.rope, scaled_and_capped=True):
     """The same model from the plain parts, float64."""
     S = len(ids)
     name = cfg.checkpoint_name
-    x = plain.embedding(ids, weights[name("embed.weight")]) * math.sqrt(cfg.hidden_size)
+    x = plain.embedding(ids, weights[name("embed.weight")])
+    if scaled_and_capped:
+        x = x * math.sqrt(cfg.hidden_size)
     for layer in range(cfg.layers):
         p = f"layers.{layer}."
         h = plain.rms_norm(x, weights[name(p + "norm1.weight")], 1e-5)
         q = plain.linear(h, weights[name(p + "mixer.q_proj.weight")]).reshape(S, cfg.heads, cfg.head_dim)
         k = plain.linear(h, weights[name(p + "mixer.k_proj.weight")]).reshape(S, 1, cfg.head_dim)
         v = plain.linear(h, weights[name(p + "mixer.v_proj.weight")]).reshape(S, 1, cfg.head_dim)
-        q = plain.rope(plain.rms_norm(q, weights[name(p + "mixer.q_norm.weight")], 1e-5), range(S), 1e4)
-        k = plain.rope(plain.rms_norm(k, weights[name(p + "mixer.k_norm.weight")], 1e-5), range(S), 1e4)
+        q = rope(plain.rms_norm(q, weights[name(p + "mixer.q_norm.weight")], 1e-5), range(S), 1e4)
+        k = rope(plain.rms_norm(k, weights[name(p + "mixer.k_norm.weight")], 1e-5), range(S), 1e4)
         x = x + plain.linear(plain.attention(q, k, v).reshape(S, -1),
                              weights[name(p + "mixer.o_proj.weight")])
         h = plain.rms_norm(x, weights[name(p + "norm2.weight")], 1e-5)
@@ -102,7 +104,7 @@ def toy_skeleton_oracle(cfg, weights, ids):
                              weights[name(p + "ffn.down_proj.weight")])
     logits = plain.linear(plain.rms_norm(x, weights[name("final_norm.weight")], 1e-5),
                           weights[name("embed.weight")])
-    return cfg.cap * torch.tanh(logits / cfg.cap)
+    return cfg.cap * torch.tanh(logits / cfg.cap) if scaled_and_capped else logits
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -143,6 +145,70 @@ def test_an_architecture_with_a_model_class_of_its_own(tmp_path, dtype):
         unregister_architecture("ToySkeletonForCausalLM")
     with pytest.raises(KeyError):
         ei.load_model(folder, dtype=dtype)
+
+
+# ---------------------------------------------------------------------------
+# an architecture whose checkpoints rotate neighbouring elements (2j, 2j + 1) instead of the
+# halves (j, j + d/2): no kernel and no position part of its own.  A query and a key give the
+# same score when both are permuted alike, so the architecture's model factory reorders the
+# rows of its q and k projections (and the per-head norm weights) once, when the model is built.
+@dataclass(frozen=True)
+class ToyNeighbourPairsConfig(ToySkeletonConfig):
+    architecture = "ToyNeighbourPairsForCausalLM"
+
+
+def neighbour_pairs_factory(spec, params, dtype, device):
+    from edge_infer_amd.engine.model import DecoderModel
+    d = spec.layers[0].mixer.head_dim
+    order = torch.cat([torch.arange(0, d, 2), torch.arange(1, d, 2)])    # evens, then odds
+
+    def per_head(rows):
+        return rows.reshape(-1, d, *rows.shape[1:])[:, order].reshape(rows.shape)
+
+    ordered = dict(params)
+    for name, tensor in params.items():
+        if name.endswith(("mixer.q_proj.weight", "mixer.k_proj.weight")):
+            ordered[name] = per_head(tensor)
+        elif name.endswith(("mixer.q_norm.weight", "mixer.k_norm.weight")):
+            ordered[name] = tensor[order]
+    return DecoderModel(spec, ordered, dtype, device)
+
+
+def neighbour_pair_rope(x, positions, theta):
+    """x [S, heads, d]: elements (2j, 2j + 1) of a head as one complex number, multiplied by
+    e^(i p theta^(-2j/d)) at position p."""
+    S, heads, d = x.shape
+    p = torch.tensor(list(positions), dtype=torch.float64)
+    frequency = theta ** (-torch.arange(0, d, 2, dtype=torch.float64) / d)
+    turn = torch.polar(torch.ones(S, d // 2, dtype=torch.float64), p[:, None] * frequency[None])
+    z = torch.view_as_complex(x.double().reshape(S, heads, d // 2, 2).contiguous()) * turn[:, None]
+    return torch.view_as_real(z).reshape(S, heads, d)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_checkpoint_that_rotates_neighbouring_elements(tmp_path, dtype):
+    import edge_infer_amd as ei
+    from edge_infer_amd.config import register_architecture, unregister_architecture
+    from safetensors.torch import load_file
+    register_architecture(ToyNeighbourPairsConfig.architecture, ToyNeighbourPairsConfig,
+                          model_factory=neighbour_pairs_factory)
+    try:
+        cfg = ToyNeighbourPairsConfig(max_positions=512)
+        folder = ei.write_model_folder(tmp_path / "pairs", cfg, seed=12)
+        weights = {k: v.double() for k, v in load_file(str(folder / "model.safetensors")).items()}
+        ids = random_ids(cfg.vocab_size, 300, 6)
+        want = toy_skeleton_oracle(cfg, weights, ids, rope=neighbour_pair_rope,
+                                   scaled_and_capped=False)
+        halves = toy_skeleton_oracle(cfg, weights, ids, scaled_and_capped=False)
+        assert (want - halves).abs().max() > 0.05 * want.abs().max(), "the pairing was meant to matter"
+        model = ei.load_model(folder, dtype=dtype)
+        session = ei.Session(model, max_tokens=512, max_seqs=2)
+        slot = session.begin()
+        rows = [session.step([(slot, ids[:270], list(range(270)))])]
+        rows += [session.step([(slot, [token], [0])]) for token in ids[270:]]
+        assert_close(dtype, torch.cat(rows), want, f"{dtype} neighbouring pairs")
+    finally:
+        unregister_architecture(ToyNeighbourPairsConfig.architecture)
 
 
 # ---------------------------------------------------------------------------
