@@ -85,65 +85,6 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
   const int head0 = g * G + hb * GB;               // first query head of this block
   const int heads_here = min(GB, G - hb * GB);
 
-  const int lo_key = window > 0 ? max(0, pos - window + 1) : 0;
-  const int first_tile = lo_key / kTile, last_tile = pos / kTile;
-  const int total_tiles = last_tile - first_tile + 1;
-  // slices are cut at page boundaries so that they do not depend on the tile size
-  const int lo_page = lo_key / EI_PAGE, hi_page = pos / EI_PAGE;
-  const int pages = hi_page - lo_page + 1;
-  // A slice is the same number of pages for every sequence of the step: the longest one's
-  // share (`longest`: the most tokens any sequence holds, read on the device so that a captured
-  // step follows it).  Sequences of unequal lengths then give blocks of about equal work, and
-  // the later slices of a short sequence are empty.  Without it (or with a window, where the
-  // ranges start at different pages) every sequence is cut into n_splits equal parts.
-  int per = (pages + n_splits - 1) / n_splits;
-  if (longest != nullptr && window <= 0) {
-    const int most_pages = (*longest + EI_PAGE - 1) / EI_PAGE;
-    per = max(1, (most_pages + n_splits - 1) / n_splits);
-  }
-  const int tile_begin = max(first_tile, (lo_page + split * per) * (EI_PAGE / kTile));
-  // (the last slice takes whatever is left, so that no key is lost should `longest` be short)
-  const int tile_end = split == n_splits - 1
-                           ? last_tile + 1
-                           : min(last_tile + 1, (lo_page + (split + 1) * per) * (EI_PAGE / kTile));
-  (void)total_tiles;
-
-  const int ks = lane / LPR, dc = lane % LPR;       // value rows: key sub-index, 8-wide chunk
-
-  // A tile of 16 keys in registers.  keys: A operand, lane (key r16, c) holds
-  // k[key][j*32 + c*8 .. +8]; values: lane (ks, dc) holds v[key0 + i*KPI + ks][dc*8 .. +8].
-  bf16x8 k_reg[DJ];
-  uint4 v_reg[VI];
-  auto page_of = [&](const int tile) {
-    return page_table[static_cast<size_t>(seq) * table_width + tile * kTile / EI_PAGE];
-  };
-  auto fetch = [&](const int tile, const int phys) {
-    const int key0 = tile * kTile;
-    const size_t page_base = (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
-    const int in_page = key0 % EI_PAGE;
-    const bf16_t* kp = k_pages + page_base + static_cast<size_t>(in_page + r16) * D + c * 8;
-#pragma unroll
-    for (int j = 0; j < DJ; ++j) k_reg[j] = *reinterpret_cast<const bf16x8*>(kp + j * 32);
-    const bf16_t* vp = v_pages + page_base + static_cast<size_t>(in_page + ks) * D + dc * 8;
-#pragma unroll
-    for (int i = 0; i < VI; ++i) {
-      // read once and whole lines at a time: not kept in the caches (the keys above are
-      // fetched in 64-byte pieces, two instructions a line, and do better cached)
-      const u32x4_t raw = __builtin_nontemporal_load(
-          reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(i) * KPI * D));
-      v_reg[i] = uint4{raw.x, raw.y, raw.z, raw.w};
-    }
-  };
-  // The page of a tile is looked up while the tile before it is worked on, the first one's
-  // before the block makes its queries (PREP).  Blocks of one or two heads also ask for their
-  // first tile there, so that the two waits for memory run side by side; with more heads the
-  // registers that would hold it across PREP cost a wave of every SIMD.  (A page the window
-  // has released, phys < 0, is all masked: nothing is fetched or computed for it.)
-  constexpr bool EARLY = GB <= 2;
-  int tile = tile_begin + wave;
-  int phys = tile < tile_end ? page_of(tile) : -1;
-  if (EARLY && tile < tile_end && phys >= 0) fetch(tile, phys);
-
   // PREP: rows 0..GB-1 the block's query heads, row GB the new key, row GB+1 the new value,
   // normed, rotated and rounded.  A wave takes a head at a time, a lane the pair (i, i + D/2):
   // every load of a head is on its way before the first is used, and nothing but the final
@@ -243,19 +184,64 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     q_reg[j] = *reinterpret_cast<bf16x8*>(&z);
   }
 
+  const int lo_key = window > 0 ? max(0, pos - window + 1) : 0;
+  const int first_tile = lo_key / kTile, last_tile = pos / kTile;
+  const int total_tiles = last_tile - first_tile + 1;
+  // slices are cut at page boundaries so that they do not depend on the tile size
+  const int lo_page = lo_key / EI_PAGE, hi_page = pos / EI_PAGE;
+  const int pages = hi_page - lo_page + 1;
+  // A slice is the same number of pages for every sequence of the step: the longest one's
+  // share (`longest`: the most tokens any sequence holds, read on the device so that a captured
+  // step follows it).  Sequences of unequal lengths then give blocks of about equal work, and
+  // the later slices of a short sequence are empty.  Without it (or with a window, where the
+  // ranges start at different pages) every sequence is cut into n_splits equal parts.
+  int per = (pages + n_splits - 1) / n_splits;
+  if (longest != nullptr && window <= 0) {
+    const int most_pages = (*longest + EI_PAGE - 1) / EI_PAGE;
+    per = max(1, (most_pages + n_splits - 1) / n_splits);
+  }
+  const int tile_begin = max(first_tile, (lo_page + split * per) * (EI_PAGE / kTile));
+  // (the last slice takes whatever is left, so that no key is lost should `longest` be short)
+  const int tile_end = split == n_splits - 1
+                           ? last_tile + 1
+                           : min(last_tile + 1, (lo_page + (split + 1) * per) * (EI_PAGE / kTile));
+  (void)total_tiles;
+
   float m_run = kLowest, l_run = 0.f;              // state of head r16 (same in all four c)
   float acc[GB][8];
 #pragma unroll
   for (int h = 0; h < GB; ++h)
 #pragma unroll
     for (int e = 0; e < 8; ++e) acc[h][e] = 0.f;
-  // One tile of 16 keys, fetched before.  OWN: the tile holds the position itself and the
-  // block has made its key and value (PREP): they come from LDS.  That case has code of its
-  // own, so that in every other tile the score product waits for the keys alone and not for a
-  // patch.
+  const int ks = lane / LPR, dc = lane % LPR;       // value rows: key sub-index, 8-wide chunk
+
+  // One tile of 16 keys.  OWN: the tile holds the position itself and the block has made its
+  // key and value (PREP): they come from LDS.  That case has code of its own, so that in
+  // every other tile the score product waits for the keys alone and not for a patch.
   auto process = [&](const int tile, auto own_tag) {
     constexpr bool OWN = decltype(own_tag)::value;
     const int key0 = tile * kTile;
+    const int phys = page_table[static_cast<size_t>(seq) * table_width + key0 / EI_PAGE];
+    if (phys < 0) return;                          // released by the window: all masked
+    const size_t page_base = (static_cast<size_t>(phys) * nkv + g) * EI_PAGE * D;
+    const int in_page = key0 % EI_PAGE;
+    // keys: A operand, lane (key r16, c) holds k[key][j*32 + c*8 .. +8]
+    bf16x8 k_reg[DJ];
+    const bf16_t* kp = k_pages + page_base + static_cast<size_t>(in_page + r16) * D + c * 8;
+#pragma unroll
+    for (int j = 0; j < DJ; ++j) k_reg[j] = *reinterpret_cast<const bf16x8*>(kp + j * 32);
+    // values: lane (ks, dc) holds v[key0 + i*KPI + ks][dc*8 .. +8]
+    uint4 v_reg[VI];
+    const bf16_t* vp = v_pages + page_base + static_cast<size_t>(in_page + ks) * D + dc * 8;
+#pragma unroll
+    for (int i = 0; i < VI; ++i)
+    {
+      // read once and whole lines at a time: not kept in the caches (the keys above are
+      // fetched in 64-byte pieces, two instructions a line, and do better cached)
+      const u32x4_t raw = __builtin_nontemporal_load(
+          reinterpret_cast<const u32x4_t*>(vp + static_cast<size_t>(i) * KPI * D));
+      v_reg[i] = uint4{raw.x, raw.y, raw.z, raw.w};
+    }
     if constexpr (OWN) {                           // the position's own key and value
       if (key0 + r16 == pos) {
 #pragma unroll
@@ -325,19 +311,11 @@ attn_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pa
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   };
-  while (tile < tile_end) {
-    const int next = tile + W;
-    const int phys_next = next < tile_end ? page_of(next) : -1;
-    if (phys >= 0) {
-      if (!EARLY) fetch(tile, phys);
-      if (PREP && own_key && tile == last_tile)
-        process(tile, std::integral_constant<bool, PREP>{});
-      else
-        process(tile, std::false_type{});
-    }
-    tile = next;
-    phys = phys_next;
-    if (EARLY && tile < tile_end && phys >= 0) fetch(tile, phys);
+  for (int tile = tile_begin + wave; tile < tile_end; tile += W) {
+    if (PREP && own_key && tile == last_tile)
+      process(tile, std::integral_constant<bool, PREP>{});
+    else
+      process(tile, std::false_type{});
   }
 
   // sum the partial outputs of the KPI key sub-groups inside the wave
