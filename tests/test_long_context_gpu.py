@@ -64,11 +64,12 @@ def test_a_prompt_of_4500_tokens_whole(models, oracle, dtype):
     slot = session.begin()
     logits = session.step([(slot, ids, places)])
     assert_close(dtype, logits, oracle(ids)[places], f"{dtype} 4,500 tokens whole")
-    # the same sequence in three portions of unequal size, the middle one of two tokens (the
-    # smallest item of the prompt path), gives the same rows
+    # the same sequence in portions of unequal size, two of them of two tokens (the smallest
+    # item of the prompt path), one inside a page and one across the border of the first page
+    # (positions 63 and 64), gives the same rows
     session.end(slot)
     slot = session.begin()
-    cuts = [0, 1500, 1502, 4500]
+    cuts = [0, 63, 65, 1500, 1502, 4500]
     rows = []
     for begin, end in zip(cuts, cuts[1:]):
         want = [p - begin for p in places if begin <= p < end]
