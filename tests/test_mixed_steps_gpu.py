@@ -231,3 +231,90 @@ def test_two_sessions_of_one_model_interleaved(fixtures, dtype):
         rows = torch.cat(got[i])
         assert_close(dtype, rows, refs[i][cuts[i] - 1:cuts[i] - 1 + rows.shape[0]],
                      f"{dtype} session {i}")
+
+
+# ---------------------------------------------------------------------------
+# Schedules nobody thought of: drawn from a seeded generator
+def random_schedule(seed, max_seqs, longest, n_requests=14, n_steps=70):
+    """(lengths, steps): requests of random lengths begin whenever a slot is free, each step
+    takes one token or a portion of 2 to 70 tokens of some of the live requests (the others
+    sit the step out), wants the last row, all rows, none or a few of them, and requests leave
+    when their tokens are used up or, now and then, earlier.  Every step mixes what it likes."""
+    import random
+    rng = random.Random(seed)
+    lengths, steps = [], []
+    at = {}                                                    # live request -> tokens brought
+    while len(steps) < n_steps and (at or len(lengths) < n_requests):
+        while len(at) < max_seqs and len(lengths) < n_requests and (not at or rng.random() < 0.3):
+            lengths.append(rng.choice([n for n in (2, 3, 17, 63, 64, 65, 66, 100, 128, 129, 190, 257)
+                                       if n <= longest]))
+            at[len(lengths) - 1] = 0
+        entries, ended = [], []
+        for request in sorted(at, key=lambda r: rng.random()):     # entries in any order
+            left = lengths[request] - at[request]
+            if entries and rng.random() < 0.15:
+                continue                                           # sits this step out
+            count = 1
+            if left >= 2 and (at[request] == 0 or rng.random() < 0.3):
+                count = rng.randint(2, min(left, 70))
+            start = at[request]
+            choice = rng.random()
+            if choice < 0.5:
+                places = [start + count - 1]
+            elif choice < 0.7:
+                places = list(range(start, start + count))
+            elif choice < 0.8:
+                places = []
+            else:
+                places = sorted(rng.sample(range(start, start + count), min(count, 3)))
+            entries.append((request, start, start + count, places))
+            at[request] += count
+            if at[request] == lengths[request] or rng.random() < 0.02:
+                ended.append(request)
+        for request in ended:
+            del at[request]
+        steps.append((entries, ended))
+    return lengths, steps
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("which,seed", [("A", 1), ("B", 2), ("long", 3), ("B", 4)])
+def test_schedules_drawn_at_random(tmp_path, which, seed, dtype):
+    """Every row that a drawn schedule returns against the plain implementation: slots are
+    given back and taken again in any order, sequences idle, prompts come in portions of any
+    size beside decoding sequences.  The cache starts full of NaN."""
+    import edge_infer_amd as ei
+    max_seqs = 5
+    shape = LONG if which == "long" else CONFIGS[which]
+    lengths, steps = random_schedule(seed, max_seqs, min(257, shape["max_position_embeddings"]))
+    assert len(lengths) >= 10 and any(ended for _, ended in steps)
+    vocab = shape["vocab_size"]
+    if which == "long":
+        folder, close = make_long_folder(tmp_path), assert_close_long
+    else:
+        folder, close = make_folder(which, tmp_path), assert_close
+    requests = [random_ids(vocab, n, 900 + 31 * seed + i) for i, n in enumerate(lengths)]
+    cfg, weights = plain.read_folder(folder)
+    refs = [plain.forward(weights, cfg, ids) for ids in requests]
+    session = ei.Session(ei.load_model(folder, dtype=dtype), max_tokens=max_seqs * 320,
+                         max_seqs=max_seqs)
+    for tensor in session.cache.kv_k + session.cache.kv_v:
+        tensor.fill_(float("nan"))
+    slots, seen_slots = {}, []
+    collected = Collected(dtype, close, refs, f"drawn {which} {seed} {dtype}")
+    for number, (entries, ended) in enumerate(steps):
+        for request, start, _, _ in entries:
+            if request not in slots:
+                assert start == 0
+                slots[request] = session.begin()
+                seen_slots.append(slots[request])
+        logits = session.step([(slots[request], requests[request][start:stop],
+                                [place - start for place in places])
+                               for request, start, stop, places in entries])
+        collected.step(number, entries, logits)
+        for request in ended:
+            session.end(slots.pop(request))
+    collected.finish()
+    for slot in slots.values():
+        session.end(slot)
+    assert len(set(seen_slots)) <= max_seqs < len(seen_slots), "slots were meant to be used again"
